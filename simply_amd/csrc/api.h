@@ -270,7 +270,8 @@ int paged_attention_generic(const void* q, int dtype, int64_t q_stride, const vo
                             const int* block_table, int table_stride, const int* token_seq, const int* positions,
                             void* out, int64_t out_stride, int T, int H, int Kh, int hd, int page_size, int window,
                             float soft_cap, hipStream_t stream, int hd_v = 0, float scale = 1.f,
-                            const void* sinks = nullptr, int sinks_dtype = 0);
+                            const void* sinks = nullptr, int sinks_dtype = 0, int maps = 1, int values_in_keys = 0,
+                            int differential = 0, float lambda = 0.f, float eps = 0.f, float mult = 1.f);
 }  // namespace sa
 
 extern "C" {
@@ -283,6 +284,18 @@ int sa_paged_attention_sink(const void* q, int dtype, int64_t q_stride, const vo
                             void* out, int64_t out_stride, int T, int H, int Kh, int hd, int hd_v, int page_size,
                             int window, float soft_cap, float scale, const void* sinks, int sinks_dtype,
                             hipStream_t stream);
+
+// Attention as sa_paged_attention_sink (no sinks, no cap) with `maps` (1 or 2) score maps per query head: a query row
+// holds H * maps vectors of hd entries (head by head, map by map), a key row maps * hd entries (key pages
+// [num_pages, Kh, page_size, maps * hd]); every map is a softmax of its own over the same values.
+// differential (maps == 2): out [T, H * hd_v] = (a_1 - lambda a_2) / sqrt(mean(.^2) + eps) * mult per head, a_m the
+// maps' results; else out [T, H * maps * hd_v] holds every map's result.
+// values_in_keys: there are no value pages (v_pages is not read); a key's value is the first hd_v entries of its row.
+int sa_paged_attention_maps(const void* q, int dtype, int64_t q_stride, const void* k_pages, const void* v_pages,
+                            const int* block_table, int table_stride, const int* token_seq, const int* positions,
+                            void* out, int64_t out_stride, int T, int H, int Kh, int hd, int hd_v, int page_size,
+                            int window, float scale, int maps, int values_in_keys, int differential, float lambda,
+                            float eps, float mult, hipStream_t stream);
 
 // residual += mult * norm(y; w) (w null: + mult * y; y null: nothing is added), then, if out is not null, out = the
 // residual in out's type: the sum of a block that norms what a part returns, and the hand-over to a next part that
@@ -309,6 +322,50 @@ int sa_qk_norm_rope_cache_write(void* proj, int dtype, int64_t row_stride, const
                                 int rot_dims, float eps, float q_mult, const void* v_first, int64_t v_first_stride,
                                 const void* lambda, int lambda_dtype, const int64_t* slot_mapping, void* k_pages,
                                 void* v_pages, int T, int H, int K, int dk, int dv, int page_size, hipStream_t stream);
+
+// residual += mult * y (y null: nothing is added), then out = residual / sqrt(mean(residual^2) + eps) * (w + plus_one):
+// the sum of a block whose parts read normed input, with the norm in front of the next part.  Rows of up to 8192.
+int sa_residual_add_next_norm(const void* y, int y_dtype, int64_t y_stride, float mult, float* residual, const void* w,
+                              int w_dtype, float eps, int plus_one, void* out, int out_dtype, int T, int D,
+                              hipStream_t stream);
+
+// On fused projection rows [H * dk queries | K * dk keys | K * dv values | ...]: every query and key vector is cut into
+// `sub` equal parts; in each part the first *_norm_dims entries are divided by sqrt(mean of their squares + eps) and
+// multiplied by *_weight [>= *_norm_dims] (null: no norm), then the entries [*_rot_at, *_rot_at + rot_dims) turn in
+// neighbouring pairs (2p, 2p + 1) by position * freq[p], cos and sin times rot_mult.  Queries go back in place, keys
+// into key pages [num_pages, K, page_size, dk], values (dv > 0) into value pages [num_pages, K, dv, page_size].
+// k_pages null: nothing is written (then K is best 0).
+int sa_norm_rope_cache_write(void* proj, int dtype, int64_t row_stride, const int* positions, const float* freq,
+                             int rot_dims, float rot_mult, const void* q_weight, int q_norm_dims, int q_rot_at,
+                             const void* k_weight, int k_norm_dims, int k_rot_at, int w_dtype, float eps, int sub,
+                             const int64_t* slot_mapping, void* k_pages, void* v_pages, int T, int H, int K, int dk,
+                             int dv, int page_size, hipStream_t stream);
+
+// y[t, c] = act(sum_j taps[c, j] (x[t - (n - 1 - j), c] + in_bias[c]) + out_bias[c]), act silu or none, as
+// sa_short_conv_silu below; either bias may be null; the tails hold x + in_bias.  Biases are of bias_dtype.
+int sa_short_conv(const void* x, int x_dtype, int64_t x_stride, const void* in_bias, const void* taps, int taps_dtype,
+                  int num_taps, const void* out_bias, int bias_dtype, int silu, float* tails, int64_t tail_stride,
+                  const int* seq_meta, int num_seqs, int max_q_len, float* y, int C, int update_tails,
+                  hipStream_t stream);
+
+// A product per head: out[t, h, o] = sum_i w[h][o][i] x[t, h, i] for o < O (w [H, O, I], row-major), summed in 32-bit
+// in the order of i.  x rows hold the heads x_head_stride apart, out rows out_head_stride apart.  tail > 0: the `tail`
+// entries behind a head's I inputs are copied behind its O outputs.  gate (null: none): one number per token and head,
+// gate[t * gate_stride + h]; the head's outputs are multiplied by sigmoid(gate).
+int sa_head_product(const void* x, int x_dtype, int64_t x_stride, int64_t x_head_stride, const void* w, int w_dtype,
+                    void* out, int out_dtype, int64_t out_stride, int64_t out_head_stride, int T, int H, int I, int O,
+                    int tail, const void* gate, int gate_dtype, int64_t gate_stride, hipStream_t stream);
+
+// The real-gated linear recurrence over each request's tokens (seq_meta [S, 4]: state slot, first row, rows, first
+// position), channel by channel, from and into state[slot] [C] float32:
+//   r = sigmoid(gr + r_bias), i = sigmoid(gi + i_bias), a = exp(-c r softplus(lam)),
+//   S <- a S + sqrt(1 - a^2) i u,   out = S * gelu_tanh(y + y_bias)
+// u [T, C] float32; gates [T, C / block] x [gr (block) | gi (block)] float32 (what sa_head_product leaves for the two
+// stacked gate matrices of every block); y rows of the activation type; biases and lam of vec_dtype.
+int sa_rglru_scan(const float* u, const float* gates, int block, const void* r_bias, const void* i_bias, const void* lam,
+                  int vec_dtype, float c, const void* y, int y_dtype, int64_t y_stride, const void* y_bias,
+                  float* state, int64_t state_stride, const int* seq_meta, int num_seqs, void* out, int out_dtype,
+                  int C, hipStream_t stream);
 
 // y[t, c] = silu(sum_j taps[c, j] x[t - (n - 1 - j), c]) over each request's tokens (seq_meta [S, 4]: state slot,
 // first row, rows, first position), with the inputs before the step's first row taken from tails[slot]

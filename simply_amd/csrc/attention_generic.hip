@@ -13,6 +13,15 @@
 // Scores -> cap -> mask -> softmax -> values as in simply/model_lib.py:611-638
 // and simply/kernels/ragged_paged_attention.py:222-249; query head h reads
 // key/value head h / G (simply/kernels/ragged_paged_attention.py:214-215).
+//
+// Three options for mixers that are not plain softmax attention:
+//   maps (M > 1)     every query head has M score maps over the same values: its query row is M vectors of hd
+//                    entries, a key row M * hd entries (one key vector per map); each map is a softmax of its own.
+//                    To the kernel a map is one more query head ("virtual head" g = head * M + map).
+//   differential     (M == 2) a head's result is (a_1 - lambda a_2) / sqrt(mean(.^2) + eps) * mult over its values,
+//                    with a_m the maps' results; otherwise every map's result is written, map by map.
+//   values_in_keys   there are no value pages: a key's value is the first hd_v entries of its key row (a latent that
+//                    is scored as it is and read as it is).
 #include "api.h"
 #include "common.h"
 
@@ -22,13 +31,22 @@ constexpr int kChunk = 64;     // keys per chunk
 constexpr int kThreads = 256;  // 4 waves
 constexpr int kMaxDimsPerThread = 2;  // head sizes up to 512
 
-template <typename T>
+struct AttentionOptions {
+  int values_in_keys = 0;
+  int differential = 0;
+  float lambda = 0.f, eps = 0.f, mult = 1.f;
+};
+
+// G: query vectors per key/value head (heads times maps); hd: entries of one of them.
+template <typename T, int M>
 __global__ __launch_bounds__(kThreads) void paged_attention_generic_kernel(
     const T* __restrict__ q, int64_t q_stride, const T* __restrict__ k_pages, const T* __restrict__ v_pages,
     const int* __restrict__ block_table, int table_stride, const int* __restrict__ token_seq,
     const int* __restrict__ positions, T* __restrict__ out, int64_t out_stride, int Kh, int G, int hd, int hd_v,
-    int page_size, int window, float soft_cap, float scale, const void* __restrict__ sinks, int sinks_dtype) {
+    int page_size, int window, float soft_cap, float scale, const void* __restrict__ sinks, int sinks_dtype,
+    AttentionOptions opt) {
   extern __shared__ float smem[];
+  __shared__ float red_s[16];
   float* q_s = smem;                      // [G][hd]
   float* s_s = q_s + G * hd;              // [G][kChunk] scores, then probabilities
   float* m_s = s_s + G * kChunk;          // [G] running maximum
@@ -37,7 +55,8 @@ __global__ __launch_bounds__(kThreads) void paged_attention_generic_kernel(
   int* page_s = reinterpret_cast<int*>(a_s + G);  // [kChunk] page of each key of the chunk
 
   const int t = blockIdx.x, kh = blockIdx.y, tid = threadIdx.x;
-  const bool tiled = keys_tiled(page_size, hd);
+  const int hd_k = M * hd;   // entries of a key row
+  const bool tiled = keys_tiled(page_size, hd_k);
   const int seq = token_seq[t];
   const int pos = positions[t];
   const int hi = pos + 1;
@@ -79,13 +98,15 @@ __global__ __launch_bounds__(kThreads) void paged_attention_generic_kernel(
         for (int g = 0; g < 8; ++g) dot[g] = 0.f;
         if (valid) {
           const int key = c0 + j;
-          const T* kp = k_pages + (static_cast<size_t>(page_s[j]) * Kh + kh) * page_size * hd;
+          const T* kp = k_pages + (static_cast<size_t>(page_s[j]) * Kh + kh) * page_size * hd_k;
           const int kin = key % page_size;
           for (int d = part; d < hd; d += 4) {
-            const float kv = to_float(kp[key_index(tiled, page_size, hd, kin, d)]);
+            float kv[M];   // the key vector of every map (g0 is a multiple of M: head g's map is g % M)
+#pragma unroll
+            for (int m = 0; m < M; ++m) kv[m] = to_float(kp[key_index(tiled, page_size, hd_k, kin, m * hd + d)]);
 #pragma unroll
             for (int g = 0; g < 8; ++g)
-              if (g < gn) dot[g] = fmaf(q_s[(g0 + g) * hd + d], kv, dot[g]);
+              if (g < gn) dot[g] = fmaf(q_s[(g0 + g) * hd + d], kv[g % M], dot[g]);
           }
         }
 #pragma unroll
@@ -133,7 +154,10 @@ __global__ __launch_bounds__(kThreads) void paged_attention_generic_kernel(
           for (int j = jlo; j < jhi; ++j) {
             const int key = c0 + j;
             const float v = to_float(
-                v_pages[((static_cast<size_t>(page_s[j]) * Kh + kh) * hd_v + d) * page_size + key % page_size]);
+                opt.values_in_keys
+                    ? k_pages[(static_cast<size_t>(page_s[j]) * Kh + kh) * page_size * hd_k +
+                              key_index(tiled, page_size, hd_k, key % page_size, d)]
+                    : v_pages[((static_cast<size_t>(page_s[j]) * Kh + kh) * hd_v + d) * page_size + key % page_size]);
 #pragma unroll
             for (int g = 0; g < 8; ++g)
               if (g < gn) acc[s][g] = fmaf(s_s[(g0 + g) * kChunk + j], v, acc[s][g]);
@@ -141,6 +165,37 @@ __global__ __launch_bounds__(kThreads) void paged_attention_generic_kernel(
         }
       }
       __syncthreads();
+    }
+    if (M == 2 && opt.differential) {
+      // heads g0 / 2 .. : o = a_1 - lambda a_2, divided by its root mean square over the head's values, times mult
+      float o[kMaxDimsPerThread][4], ss[4];
+#pragma unroll
+      for (int p = 0; p < 4; ++p) ss[p] = 0.f;
+#pragma unroll
+      for (int s = 0; s < kMaxDimsPerThread; ++s) {
+        const int d = tid + s * kThreads;
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+          o[s][p] = 0.f;
+          if (d < hd_v && 2 * p + 1 < gn) {
+            o[s][p] = acc[s][2 * p] / l_s[g0 + 2 * p] - opt.lambda * (acc[s][2 * p + 1] / l_s[g0 + 2 * p + 1]);
+            ss[p] = fmaf(o[s][p], o[s][p], ss[p]);
+          }
+        }
+      }
+#pragma unroll
+      for (int p = 0; p < 4; ++p) {
+        if (2 * p + 1 >= gn) break;   // (uniform over the workgroup)
+        const float r = opt.mult / sqrtf(block_sum(ss[p], red_s) / static_cast<float>(hd_v) + opt.eps);
+#pragma unroll
+        for (int s = 0; s < kMaxDimsPerThread; ++s) {
+          const int d = tid + s * kThreads;
+          if (d < hd_v)
+            out[static_cast<size_t>(t) * out_stride + static_cast<size_t>((kh * G + g0) / 2 + p) * hd_v + d] =
+                from_float<T>(o[s][p] * r);
+        }
+      }
+      continue;
     }
 #pragma unroll
     for (int s = 0; s < kMaxDimsPerThread; ++s) {
@@ -160,13 +215,49 @@ __global__ __launch_bounds__(kThreads) void paged_attention_generic_kernel(
   }
 }
 
+template <int M>
+static void launch_generic(const void* q, int dtype, int64_t q_stride, const void* k_pages, const void* v_pages,
+                           const int* block_table, int table_stride, const int* token_seq, const int* positions,
+                           void* out, int64_t out_stride, int T, int Kh, int G, int hd, int hd_v, int page_size,
+                           int window, float soft_cap, float scale, const void* sinks, int sinks_dtype,
+                           AttentionOptions opt, size_t smem, hipStream_t stream) {
+  const dim3 grid(T, Kh);
+  if (dtype == kF32)
+    paged_attention_generic_kernel<float, M><<<grid, kThreads, smem, stream>>>(
+        static_cast<const float*>(q), q_stride, static_cast<const float*>(k_pages),
+        static_cast<const float*>(v_pages), block_table, table_stride, token_seq, positions, static_cast<float*>(out),
+        out_stride, Kh, G, hd, hd_v, page_size, window, soft_cap, scale, sinks, sinks_dtype, opt);
+  else
+    paged_attention_generic_kernel<bf16, M><<<grid, kThreads, smem, stream>>>(
+        static_cast<const bf16*>(q), q_stride, static_cast<const bf16*>(k_pages), static_cast<const bf16*>(v_pages),
+        block_table, table_stride, token_seq, positions, static_cast<bf16*>(out), out_stride, Kh, G, hd, hd_v, page_size,
+        window, soft_cap, scale, sinks, sinks_dtype, opt);
+}
+
 int paged_attention_generic(const void* q, int dtype, int64_t q_stride, const void* k_pages, const void* v_pages,
                             const int* block_table, int table_stride, const int* token_seq, const int* positions,
                             void* out, int64_t out_stride, int T, int H, int Kh, int hd, int page_size, int window,
                             float soft_cap, hipStream_t stream, int hd_v, float scale, const void* sinks,
-                            int sinks_dtype) {
-  const int G = H / Kh;
+                            int sinks_dtype, int maps, int values_in_keys, int differential, float lambda, float eps,
+                            float mult) {
+  const int G = H / Kh * maps;   // query vectors per key/value head
   if (hd_v <= 0) hd_v = hd;
+  if (maps != 1 && maps != 2) {
+    set_error("paged_attention: %d score maps per head (1 or 2)", maps);
+    return 1;
+  }
+  if (differential && maps != 2) {
+    set_error("paged_attention: the differential combination needs two score maps per head");
+    return 1;
+  }
+  if (maps > 1 && sinks != nullptr) {
+    set_error("paged_attention: sinks and several score maps do not combine");
+    return 1;
+  }
+  if (values_in_keys && hd_v > maps * hd) {
+    set_error("paged_attention: %d values cannot be read from key rows of %d entries", hd_v, maps * hd);
+    return 1;
+  }
   if (hd_v > kThreads * kMaxDimsPerThread) {
     set_error("paged_attention: value size %d is above the largest supported (%d)", hd_v, kThreads * kMaxDimsPerThread);
     return 1;
@@ -174,21 +265,24 @@ int paged_attention_generic(const void* q, int dtype, int64_t q_stride, const vo
   const size_t smem = sizeof(float) * (static_cast<size_t>(G) * hd + static_cast<size_t>(G) * kChunk + 3 * G) +
                       sizeof(int) * kChunk;
   if (smem > 64 * 1024) {
-    set_error("paged_attention: %d query heads per key head at head size %d need %zu bytes of LDS (limit 65536)", G,
+    set_error("paged_attention: %d query vectors per key head of size %d need %zu bytes of LDS (limit 65536)", G,
               hd, smem);
     return 1;
   }
-  const dim3 grid(T, Kh);
-  if (dtype == kF32)
-    paged_attention_generic_kernel<float><<<grid, kThreads, smem, stream>>>(
-        static_cast<const float*>(q), q_stride, static_cast<const float*>(k_pages),
-        static_cast<const float*>(v_pages), block_table, table_stride, token_seq, positions, static_cast<float*>(out),
-        out_stride, Kh, G, hd, hd_v, page_size, window, soft_cap, scale, sinks, sinks_dtype);
+  AttentionOptions opt;
+  opt.values_in_keys = values_in_keys;
+  opt.differential = differential;
+  opt.lambda = lambda;
+  opt.eps = eps;
+  opt.mult = mult;
+  if (maps == 2)
+    launch_generic<2>(q, dtype, q_stride, k_pages, v_pages, block_table, table_stride, token_seq, positions, out,
+                      out_stride, T, Kh, G, hd, hd_v, page_size, window, soft_cap, scale, sinks, sinks_dtype, opt, smem,
+                      stream);
   else
-    paged_attention_generic_kernel<bf16><<<grid, kThreads, smem, stream>>>(
-        static_cast<const bf16*>(q), q_stride, static_cast<const bf16*>(k_pages), static_cast<const bf16*>(v_pages),
-        block_table, table_stride, token_seq, positions, static_cast<bf16*>(out), out_stride, Kh, G, hd, hd_v, page_size,
-        window, soft_cap, scale, sinks, sinks_dtype);
+    launch_generic<1>(q, dtype, q_stride, k_pages, v_pages, block_table, table_stride, token_seq, positions, out,
+                      out_stride, T, Kh, G, hd, hd_v, page_size, window, soft_cap, scale, sinks, sinks_dtype, opt, smem,
+                      stream);
   return check_launch("paged_attention_generic");
 }
 

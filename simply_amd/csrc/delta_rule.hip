@@ -17,12 +17,15 @@ namespace sa {
 constexpr int kMaxTaps = 8;
 constexpr int kConvTokens = 16;  // tokens that one thread of the convolution walks through
 
-// y[t, c] = silu(sum_j taps[c, j] * x[t - (n - 1 - j), c]) with x before the step's first token taken from the
-// request's tail [n - 1][C] (oldest first).  A thread takes one channel and kConvTokens consecutive tokens.
-__global__ __launch_bounds__(kWave) void short_conv_silu_kernel(
+// y[t, c] = act(sum_j taps[c, j] * x[t - (n - 1 - j), c] + out_bias[c]) with x before the step's first token taken
+// from the request's tail [n - 1][C] (oldest first); act is silu (kSilu) or nothing.  With in_bias, x stands for
+// x + in_bias[c] (a projection's bias that has not been added yet; the tails hold the sums).  A thread takes one
+// channel and kConvTokens consecutive tokens.
+template <bool kSilu>
+__global__ __launch_bounds__(kWave) void short_conv_kernel(
     const void* __restrict__ x, int x_dtype, int64_t x_stride, const void* __restrict__ taps, int taps_dtype, int n,
     const float* __restrict__ tails, int64_t tail_stride, const int* __restrict__ seq_meta, float* __restrict__ y,
-    int C) {
+    int C, const void* __restrict__ in_bias, const void* __restrict__ out_bias, int bias_dtype) {
   const int* meta = seq_meta + 4 * blockIdx.y;
   const int slot = meta[0], first = meta[1], count = meta[2];
   const int j0 = blockIdx.x * kConvTokens;
@@ -32,8 +35,13 @@ __global__ __launch_bounds__(kWave) void short_conv_silu_kernel(
 #pragma unroll
   for (int i = 0; i < kMaxTaps; ++i) w[i] = i < n ? load_f(taps, taps_dtype, static_cast<size_t>(c) * n + i) : 0.f;
   const float* tail = tails + static_cast<size_t>(slot) * tail_stride;
+  const float b_in = in_bias != nullptr ? load_f(in_bias, bias_dtype, c) : 0.f;
+  const float b_out = out_bias != nullptr ? load_f(out_bias, bias_dtype, c) : 0.f;
   auto input = [&](int j) -> float {   // j: token of the request in this step; negative: before the step
-    if (j >= 0) return load_f(x, x_dtype, static_cast<size_t>(first + j) * x_stride + c);
+    if (j >= 0) {
+      const float v = load_f(x, x_dtype, static_cast<size_t>(first + j) * x_stride + c);
+      return in_bias != nullptr ? v + b_in : v;
+    }
     return tail[static_cast<size_t>(n - 1 + j) * C + c];
   };
 #pragma unroll
@@ -51,7 +59,8 @@ __global__ __launch_bounds__(kWave) void short_conv_silu_kernel(
 #pragma unroll
     for (int i = 0; i < kMaxTaps; ++i)
       if (i < n) acc = fmaf(w[i], win[i], acc);
-    y[static_cast<size_t>(first + j0 + j) * C + c] = acc / (1.f + expf(-acc));
+    if (out_bias != nullptr) acc += b_out;
+    y[static_cast<size_t>(first + j0 + j) * C + c] = kSilu ? acc / (1.f + expf(-acc)) : acc;
   }
 }
 
@@ -61,7 +70,8 @@ __global__ __launch_bounds__(kWave) void short_conv_silu_kernel(
 __global__ __launch_bounds__(kWave) void conv_tail_update_kernel(const void* __restrict__ x, int x_dtype,
                                                                  int64_t x_stride, int n, float* __restrict__ tails,
                                                                  int64_t tail_stride, const int* __restrict__ seq_meta,
-                                                                 int C) {
+                                                                 int C, const void* __restrict__ in_bias = nullptr,
+                                                                 int bias_dtype = 0) {
   const int* meta = seq_meta + 4 * blockIdx.y;
   const int slot = meta[0], first = meta[1], count = meta[2];
   const int c = blockIdx.x * kWave + threadIdx.x;
@@ -69,8 +79,14 @@ __global__ __launch_bounds__(kWave) void conv_tail_update_kernel(const void* __r
   float* tail = tails + static_cast<size_t>(slot) * tail_stride;
   for (int i = 0; i < n - 1; ++i) {
     const int j = count - (n - 1) + i;   // token of this step that becomes entry i; negative: an old entry
-    tail[static_cast<size_t>(i) * C + c] = j >= 0 ? load_f(x, x_dtype, static_cast<size_t>(first + j) * x_stride + c)
-                                                  : tail[static_cast<size_t>(n - 1 + j) * C + c];
+    float v;
+    if (j >= 0) {
+      v = load_f(x, x_dtype, static_cast<size_t>(first + j) * x_stride + c);
+      if (in_bias != nullptr) v += load_f(in_bias, bias_dtype, c);
+    } else {
+      v = tail[static_cast<size_t>(n - 1 + j) * C + c];
+    }
+    tail[static_cast<size_t>(i) * C + c] = v;
   }
 }
 
@@ -327,24 +343,36 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(const float* __restrict
 
 using namespace sa;
 
-extern "C" int sa_short_conv_silu(const void* x, int x_dtype, int64_t x_stride, const void* taps, int taps_dtype,
-                                  int num_taps, float* tails, int64_t tail_stride, const int* seq_meta, int num_seqs,
-                                  int max_q_len, float* y, int C, int update_tails, hipStream_t stream) {
+extern "C" int sa_short_conv(const void* x, int x_dtype, int64_t x_stride, const void* in_bias, const void* taps,
+                             int taps_dtype, int num_taps, const void* out_bias, int bias_dtype, int silu, float* tails,
+                             int64_t tail_stride, const int* seq_meta, int num_seqs, int max_q_len, float* y, int C,
+                             int update_tails, hipStream_t stream) {
   if (num_seqs == 0 || max_q_len == 0) return 0;
   SA_REQUIRE(num_seqs > 0 && max_q_len > 0 && C > 0 && x != nullptr && taps != nullptr &&
                  (tails != nullptr || num_taps == 1) && seq_meta != nullptr && y != nullptr,
-             "short_conv_silu: bad sizes S=%d q=%d C=%d", num_seqs, max_q_len, C);
-  SA_REQUIRE(num_taps >= 1 && num_taps <= kMaxTaps, "short_conv_silu: 1 to %d taps, got %d", kMaxTaps, num_taps);
+             "short_conv: bad sizes S=%d q=%d C=%d", num_seqs, max_q_len, C);
+  SA_REQUIRE(num_taps >= 1 && num_taps <= kMaxTaps, "short_conv: 1 to %d taps, got %d", kMaxTaps, num_taps);
   SA_REQUIRE(x_stride >= C && tail_stride >= static_cast<int64_t>(num_taps - 1) * C,
-             "short_conv_silu: a stride is below what the %d channels need", C);
-  SA_REQUIRE(num_seqs <= 65535 && (C + kWave - 1) / kWave <= 65535, "short_conv_silu: too many requests or channels");
+             "short_conv: a stride is below what the %d channels need", C);
+  SA_REQUIRE(num_seqs <= 65535 && (C + kWave - 1) / kWave <= 65535, "short_conv: too many requests or channels");
   const dim3 grid((max_q_len + kConvTokens - 1) / kConvTokens, num_seqs, (C + kWave - 1) / kWave);
-  short_conv_silu_kernel<<<grid, kWave, 0, stream>>>(x, x_dtype, x_stride, taps, taps_dtype, num_taps, tails,
-                                                     tail_stride, seq_meta, y, C);
+  if (silu)
+    short_conv_kernel<true><<<grid, kWave, 0, stream>>>(x, x_dtype, x_stride, taps, taps_dtype, num_taps, tails,
+                                                        tail_stride, seq_meta, y, C, in_bias, out_bias, bias_dtype);
+  else
+    short_conv_kernel<false><<<grid, kWave, 0, stream>>>(x, x_dtype, x_stride, taps, taps_dtype, num_taps, tails,
+                                                         tail_stride, seq_meta, y, C, in_bias, out_bias, bias_dtype);
   if (update_tails && num_taps > 1)
     conv_tail_update_kernel<<<dim3((C + kWave - 1) / kWave, num_seqs), kWave, 0, stream>>>(
-        x, x_dtype, x_stride, num_taps, tails, tail_stride, seq_meta, C);
-  return check_launch("short_conv_silu");
+        x, x_dtype, x_stride, num_taps, tails, tail_stride, seq_meta, C, in_bias, bias_dtype);
+  return check_launch("short_conv");
+}
+
+extern "C" int sa_short_conv_silu(const void* x, int x_dtype, int64_t x_stride, const void* taps, int taps_dtype,
+                                  int num_taps, float* tails, int64_t tail_stride, const int* seq_meta, int num_seqs,
+                                  int max_q_len, float* y, int C, int update_tails, hipStream_t stream) {
+  return sa_short_conv(x, x_dtype, x_stride, nullptr, taps, taps_dtype, num_taps, nullptr, 0, 1, tails, tail_stride,
+                       seq_meta, num_seqs, max_q_len, y, C, update_tails, stream);
 }
 
 extern "C" int sa_delta_prepare(float* qkv, int T, int C, int G, int dk, const void* ab, int ab_dtype, int64_t ab_stride,

@@ -96,6 +96,54 @@ static bool launch_residual_add_norm_typed(const void* y, int64_t y_stride, cons
   return true;
 }
 
+// ------------------------------------------------------------------ residual += mult * y; out = norm(residual)
+// The sum of a block that norms what its parts read (their results are added as they are, times a constant), fused
+// with the norm in front of the next part: out = h / sqrt(mean(h^2) + eps) * (w + plus_one) over the updated row h,
+// which is held in registers between the two.  y null: nothing is added.
+template <typename YT, typename OT, int NP>
+__global__ __launch_bounds__(256) void residual_add_next_norm_kernel(
+    const YT* __restrict__ y, int64_t y_stride, float mult, float* __restrict__ residual, const void* __restrict__ w,
+    int w_dtype, float eps, float plus_one, OT* __restrict__ out, int D) {
+  __shared__ float scratch[16];
+  const size_t yb = static_cast<size_t>(blockIdx.x) * y_stride, rb = static_cast<size_t>(blockIdx.x) * D;
+  float hv[NP], wv[NP];
+  float ss = 0.f;
+#pragma unroll
+  for (int p = 0; p < NP; ++p) {
+    const int d = threadIdx.x + p * 256;
+    const bool ok = d < D;
+    const float yv = (ok && y != nullptr) ? to_float(y[yb + d]) : 0.f;
+    const float h = ok ? residual[rb + d] : 0.f;
+    wv[p] = ok ? load_f(w, w_dtype, d) + plus_one : 0.f;
+    hv[p] = y != nullptr ? h + mult * yv : h;
+    if (ok && y != nullptr) residual[rb + d] = hv[p];
+    ss = fmaf(hv[p], hv[p], ss);
+  }
+  ss = block_sum(ss, scratch);
+  const float r = 1.f / sqrtf(ss / static_cast<float>(D) + eps);
+#pragma unroll
+  for (int p = 0; p < NP; ++p) {
+    const int d = threadIdx.x + p * 256;
+    if (d < D) out[rb + d] = from_float<OT>(hv[p] * r * wv[p]);
+  }
+}
+
+template <typename YT, typename OT>
+static void launch_residual_add_next_norm(const void* y, int64_t y_stride, float mult, float* residual, const void* w,
+                                          int w_dtype, float eps, float plus_one, void* out, int T, int D,
+                                          hipStream_t stream) {
+  const YT* yp = static_cast<const YT*>(y);
+  OT* op = static_cast<OT*>(out);
+  if (D <= 1024)
+    residual_add_next_norm_kernel<YT, OT, 4><<<T, 256, 0, stream>>>(yp, y_stride, mult, residual, w, w_dtype, eps, plus_one, op, D);
+  else if (D <= 2048)
+    residual_add_next_norm_kernel<YT, OT, 8><<<T, 256, 0, stream>>>(yp, y_stride, mult, residual, w, w_dtype, eps, plus_one, op, D);
+  else if (D <= 4096)
+    residual_add_next_norm_kernel<YT, OT, 16><<<T, 256, 0, stream>>>(yp, y_stride, mult, residual, w, w_dtype, eps, plus_one, op, D);
+  else
+    residual_add_next_norm_kernel<YT, OT, 32><<<T, 256, 0, stream>>>(yp, y_stride, mult, residual, w, w_dtype, eps, plus_one, op, D);
+}
+
 // ------------------------------------------------------------------ heads normed and gated
 // out[t, h, :] = (w ? x[t, h, :] / sqrt(mean(x[t, h, :]^2) + eps) * w : x[t, h, :]) * gate(g[t, h, :]),
 // gate 0: sigmoid, 1: silu.  One wave per (token, head); w [size] is shared by the heads.
@@ -217,6 +265,97 @@ __global__ __launch_bounds__(kWave) void qk_norm_rope_cache_write_kernel(
   }
 }
 
+// ------------------------------------------------------------------ queries and keys: weighted norm, then rotation
+// One wave per (token, head) of a fused projection row [H * dk queries | K * dk keys | K * dv values | ...].  A query
+// or key vector of dk entries is cut into `sub` equal parts (the score maps of a head); in every part
+//   the first norm_dims entries are divided by sqrt(mean of their squares + eps) and multiplied by w[i] (w null: not),
+//   then the entries [rot_at, rot_at + rot_dims) turn in neighbouring pairs: (u, v) at the pair p becomes
+//   rot_mult * (u cos a - v sin a, v cos a + u sin a) with a = position * freq[p].
+// Queries go back in place, keys into the key pages (rows of dk entries), values as they are into the value pages
+// (transposed); dv == 0: there are no values.  norm_dims, rot_at and w are given for queries and for keys.
+struct HeadNormRope {
+  const void* w;
+  int norm_dims, rot_at;
+};
+constexpr int kPartPerLane = 16;  // parts of up to 1024 entries
+template <typename T>
+__global__ __launch_bounds__(kWave) void norm_rope_cache_write_kernel(
+    T* __restrict__ proj, int64_t row_stride, const int* __restrict__ positions, const float* __restrict__ freq,
+    int rot_dims, float rot_mult, HeadNormRope qn, HeadNormRope kn, int w_dtype, float eps, int sub,
+    const int64_t* __restrict__ slot_mapping, T* __restrict__ k_pages, T* __restrict__ v_pages, int H, int K, int dk,
+    int dv, int page_size) {
+  const int t = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+  T* row = proj + static_cast<size_t>(t) * row_stride;
+  if (head < H + K) {
+    const bool is_q = head < H;
+    const HeadNormRope hn = is_q ? qn : kn;
+    const int ds = dk / sub;
+    const float pos = static_cast<float>(positions[t]);
+    int64_t slot = -1;
+    T* dst = nullptr;
+    bool tiled = false;
+    int koff = 0;
+    if (!is_q) {
+      if (k_pages == nullptr) return;
+      slot = slot_mapping[t];
+      if (slot < 0) return;
+      koff = static_cast<int>(slot % page_size);
+      dst = k_pages + ((slot / page_size) * K + (head - H)) * page_size * dk;
+      tiled = keys_tiled(page_size, dk);
+    }
+    for (int part = 0; part < sub; ++part) {
+      T* src = row + static_cast<size_t>(head) * dk + static_cast<size_t>(part) * ds;
+      float raw[kPartPerLane], other[kPartPerLane];
+      float ss = 0.f;
+#pragma unroll
+      for (int j = 0; j < kPartPerLane; ++j) {
+        const int i = lane + j * kWave;
+        raw[j] = other[j] = 0.f;
+        if (i < ds) {
+          raw[j] = to_float(src[i]);
+          const int e = i - hn.rot_at;
+          if (e >= 0 && e < rot_dims) other[j] = to_float(src[hn.rot_at + (e ^ 1)]);
+          if (i < hn.norm_dims) ss = fmaf(raw[j], raw[j], ss);
+        }
+      }
+      float r = 1.f;
+      if (hn.w != nullptr && hn.norm_dims > 0) {
+        ss = wave_sum(ss);
+        r = 1.f / sqrtf(ss / static_cast<float>(hn.norm_dims) + eps);
+      }
+      // (every lane has read what it needs of the part before any lane writes: the wave runs in lockstep)
+#pragma unroll
+      for (int j = 0; j < kPartPerLane; ++j) {
+        const int i = lane + j * kWave;
+        if (i >= ds) continue;
+        float v = raw[j];
+        if (hn.w != nullptr && i < hn.norm_dims) v = v * r * load_f(hn.w, w_dtype, i);
+        const int e = i - hn.rot_at;
+        if (e >= 0 && e < rot_dims) {
+          const int pi = hn.rot_at + (e ^ 1);
+          float o = other[j];
+          if (hn.w != nullptr && pi < hn.norm_dims) o = o * r * load_f(hn.w, w_dtype, pi);
+          float sn, cs;
+          sincosf(pos * freq[e >> 1], &sn, &cs);
+          sn *= rot_mult;
+          cs *= rot_mult;
+          v = (e & 1) == 0 ? v * cs - o * sn : v * cs + o * sn;
+        }
+        if (is_q) src[i] = from_float<T>(v);
+        else dst[key_index(tiled, page_size, dk, koff, part * ds + i)] = from_float<T>(v);
+      }
+    }
+    return;
+  }
+  if (v_pages == nullptr) return;
+  const int64_t slot = slot_mapping[t];
+  if (slot < 0) return;
+  const int vh = head - H - K;
+  const T* src = row + static_cast<size_t>(H + K) * dk + static_cast<size_t>(vh) * dv;
+  T* dst = v_pages + ((slot / page_size) * K + vh) * page_size * dv + slot % page_size;
+  for (int i = lane; i < dv; i += kWave) dst[static_cast<size_t>(i) * page_size] = src[i];
+}
+
 }  // namespace sa
 
 using namespace sa;
@@ -241,6 +380,30 @@ extern "C" int sa_residual_add_norm(const void* y, int y_dtype, int64_t y_stride
     residual_add_norm_kernel<<<T, 256, 0, stream>>>(y, y_dtype, y_stride, w, w_dtype, eps, plus, mult, residual, out,
                                                     out_dtype, D);
   return check_launch("residual_add_norm");
+}
+
+extern "C" int sa_residual_add_next_norm(const void* y, int y_dtype, int64_t y_stride, float mult, float* residual,
+                                         const void* w, int w_dtype, float eps, int plus_one, void* out, int out_dtype,
+                                         int T, int D, hipStream_t stream) {
+  if (T == 0) return 0;
+  SA_REQUIRE(T > 0 && D > 0 && D <= 8192 && residual != nullptr && w != nullptr && out != nullptr,
+             "residual_add_next_norm: bad sizes T=%d D=%d (rows of at most 8192), or a null pointer", T, D);
+  SA_REQUIRE(y == nullptr || y_stride >= D, "residual_add_next_norm: row stride %lld is below the width %d",
+             (long long)y_stride, D);
+  SA_REQUIRE(eps >= 0.f, "residual_add_next_norm: eps must not be negative");
+  const float plus = plus_one ? 1.f : 0.f;
+  const bool yb = y == nullptr ? out_dtype == kBF16 : y_dtype == kBF16;
+  SA_REQUIRE((y == nullptr || y_dtype == kBF16 || y_dtype == kF32) && (out_dtype == kBF16 || out_dtype == kF32),
+             "residual_add_next_norm: rows are bfloat16 or float32");
+  if (yb && out_dtype == kBF16)
+    launch_residual_add_next_norm<bf16, bf16>(y, y_stride, mult, residual, w, w_dtype, eps, plus, out, T, D, stream);
+  else if (yb)
+    launch_residual_add_next_norm<bf16, float>(y, y_stride, mult, residual, w, w_dtype, eps, plus, out, T, D, stream);
+  else if (out_dtype == kBF16)
+    launch_residual_add_next_norm<float, bf16>(y, y_stride, mult, residual, w, w_dtype, eps, plus, out, T, D, stream);
+  else
+    launch_residual_add_next_norm<float, float>(y, y_stride, mult, residual, w, w_dtype, eps, plus, out, T, D, stream);
+  return check_launch("residual_add_next_norm");
 }
 
 extern "C" int sa_gated_heads(const void* x, int x_dtype, int64_t x_stride, const void* g, int g_dtype, int64_t g_stride,
@@ -311,4 +474,42 @@ extern "C" int sa_qk_norm_rope_cache_write(void* proj, int dtype, int64_t row_st
   else
     SA_REQUIRE(false, "qk_norm_rope_cache_write: unknown dtype %d", dtype);
   return check_launch("qk_norm_rope_cache_write");
+}
+
+extern "C" int sa_norm_rope_cache_write(void* proj, int dtype, int64_t row_stride, const int* positions,
+                                        const float* freq, int rot_dims, float rot_mult, const void* q_weight,
+                                        int q_norm_dims, int q_rot_at, const void* k_weight, int k_norm_dims,
+                                        int k_rot_at, int w_dtype, float eps, int sub, const int64_t* slot_mapping,
+                                        void* k_pages, void* v_pages, int T, int H, int K, int dk, int dv,
+                                        int page_size, hipStream_t stream) {
+  if (T == 0) return 0;
+  SA_REQUIRE(T > 0 && H >= 0 && K >= 0 && H + K > 0 && dk > 0 && dv >= 0 && page_size > 0 && sub > 0,
+             "norm_rope_cache_write: bad sizes T=%d H=%d K=%d dk=%d dv=%d P=%d sub=%d", T, H, K, dk, dv, page_size, sub);
+  SA_REQUIRE(dk % sub == 0 && dk / sub <= kPartPerLane * kWave,
+             "norm_rope_cache_write: vectors of %d entries in %d parts (equal parts of at most %d)", dk, sub,
+             kPartPerLane * kWave);
+  const int ds = dk / sub;
+  SA_REQUIRE(rot_dims >= 0 && rot_dims % 2 == 0 && (rot_dims == 0 || freq != nullptr) && q_rot_at >= 0 && k_rot_at >= 0 &&
+                 q_rot_at + rot_dims <= ds && k_rot_at + rot_dims <= ds,
+             "norm_rope_cache_write: %d rotated entries do not fit into parts of %d", rot_dims, ds);
+  SA_REQUIRE(q_norm_dims >= 0 && q_norm_dims <= ds && k_norm_dims >= 0 && k_norm_dims <= ds && eps >= 0.f,
+             "norm_rope_cache_write: normed entries beyond a part, or a negative eps");
+  SA_REQUIRE(row_stride >= static_cast<int64_t>(H + K) * dk + static_cast<int64_t>(K) * dv,
+             "norm_rope_cache_write: row stride %lld is too small", (long long)row_stride);
+  SA_REQUIRE(k_pages == nullptr || (slot_mapping != nullptr && (dv == 0 || v_pages != nullptr)),
+             "norm_rope_cache_write: key pages come with slots (and value pages, if there are values)");
+  SA_REQUIRE(H + 2 * K <= 65535, "norm_rope_cache_write: too many heads");
+  const dim3 grid(T, H + K + (dv > 0 ? K : 0));
+  const HeadNormRope qn{q_weight, q_norm_dims, q_rot_at}, kn{k_weight, k_norm_dims, k_rot_at};
+  if (dtype == kF32)
+    norm_rope_cache_write_kernel<float><<<grid, kWave, 0, stream>>>(
+        static_cast<float*>(proj), row_stride, positions, freq, rot_dims, rot_mult, qn, kn, w_dtype, eps, sub,
+        slot_mapping, static_cast<float*>(k_pages), static_cast<float*>(v_pages), H, K, dk, dv, page_size);
+  else if (dtype == kBF16)
+    norm_rope_cache_write_kernel<bf16><<<grid, kWave, 0, stream>>>(
+        static_cast<bf16*>(proj), row_stride, positions, freq, rot_dims, rot_mult, qn, kn, w_dtype, eps, sub,
+        slot_mapping, static_cast<bf16*>(k_pages), static_cast<bf16*>(v_pages), H, K, dk, dv, page_size);
+  else
+    SA_REQUIRE(false, "norm_rope_cache_write: unknown dtype %d", dtype);
+  return check_launch("norm_rope_cache_write");
 }

@@ -193,6 +193,29 @@ extern "C" int sa_paged_attention_sink(const void* q, int dtype, int64_t q_strid
                                  sinks_dtype);
 }
 
+extern "C" int sa_paged_attention_maps(const void* q, int dtype, int64_t q_stride, const void* k_pages,
+                                       const void* v_pages, const int* block_table, int table_stride,
+                                       const int* token_seq, const int* positions, void* out, int64_t out_stride, int T,
+                                       int H, int Kh, int hd, int hd_v, int page_size, int window, float scale,
+                                       int maps, int values_in_keys, int differential, float lambda, float eps,
+                                       float mult, hipStream_t stream) {
+  if (T == 0) return 0;
+  SA_REQUIRE(dtype == kF32 || dtype == kBF16, "paged_attention_maps: unknown dtype %d", dtype);
+  SA_REQUIRE(T > 0 && H > 0 && Kh > 0 && hd > 0 && hd_v > 0 && page_size > 0 && maps > 0,
+             "paged_attention_maps: bad sizes T=%d H=%d K=%d hd=%d hd_v=%d P=%d maps=%d", T, H, Kh, hd, hd_v, page_size,
+             maps);
+  SA_REQUIRE(H % Kh == 0, "paged_attention_maps: %d query heads do not split over %d key heads", H, Kh);
+  SA_REQUIRE(q_stride >= static_cast<int64_t>(H) * maps * hd &&
+                 out_stride >= static_cast<int64_t>(H) * (differential ? 1 : maps) * hd_v,
+             "paged_attention_maps: row strides are below what the heads need");
+  SA_REQUIRE(window >= 0 && table_stride > 0, "paged_attention_maps: bad window or table stride");
+  SA_REQUIRE(values_in_keys || v_pages != nullptr, "paged_attention_maps: no value pages");
+  SA_REQUIRE(eps >= 0.f, "paged_attention_maps: eps must not be negative");
+  return paged_attention_generic(q, dtype, q_stride, k_pages, v_pages, block_table, table_stride, token_seq, positions,
+                                 out, out_stride, T, H, Kh, hd, page_size, window, 0.f, stream, hd_v, scale, nullptr, 0,
+                                 maps, values_in_keys, differential, lambda, eps, mult);
+}
+
 extern "C" int sa_paged_attention_decode_sink(const void* q, int64_t q_stride, const void* k_pages,
                                               const void* v_pages, const int* block_table, int table_stride,
                                               const int* seq_meta, int seq_begin, int seq_count, void* out,

@@ -726,6 +726,56 @@ def paged_attention_sink(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.
     return out
 
 
+def paged_attention_maps(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor | None, block_table: torch.Tensor,
+                         token_seq: torch.Tensor, positions: torch.Tensor, num_heads: int, *, scale: float,
+                         maps: int = 1, value_dim: int | None = None, window: int | None = None,
+                         differential: "tuple[float, float, float] | None" = None,
+                         out: torch.Tensor | None = None) -> torch.Tensor:
+    """Attention with `maps` score maps per query head, each a softmax of its own over the same values: q rows hold
+    H * maps vectors of hd entries (head by head, map by map), key pages [pages, K, P, maps * hd].  With value pages
+    [pages, K, dv, P]; v_pages None: a key's value is the first `value_dim` entries of its own row.  differential
+    (lambda, eps, mult), for two maps: returns [T, H * dv] = (a_1 - lambda a_2) / sqrt(mean(.^2) + eps) * mult per
+    head; else [T, H * maps * dv], every map's result."""
+    _dev(q, k_pages, v_pages, block_table, token_seq, positions, out)
+    q_stride = _rows(q, "paged_attention_maps: q")
+    T = q.shape[0]
+    if k_pages.dim() != 4 or not k_pages.is_contiguous() or k_pages.dtype != q.dtype:
+        raise KernelError(f"paged_attention_maps: key pages must be a contiguous 4-D tensor of {q.dtype}")
+    num_pages, Kh, page_size, row = k_pages.shape
+    if maps not in (1, 2) or row % maps:
+        raise KernelError(f"paged_attention_maps: key rows of {row} entries for {maps} maps")
+    hd = row // maps
+    if v_pages is not None:
+        dv = v_pages.shape[2]
+        if v_pages.dtype != q.dtype or not v_pages.is_contiguous() or tuple(v_pages.shape) != (num_pages, Kh, dv, page_size):
+            raise KernelError(f"paged_attention_maps: key pages {tuple(k_pages.shape)} do not go with value pages "
+                              f"{tuple(v_pages.shape)}")
+    else:
+        dv = int(value_dim or 0)
+        if not 0 < dv <= row:
+            raise KernelError(f"paged_attention_maps: {dv} values out of key rows of {row} entries")
+    if q.shape[1] < num_heads * maps * hd:
+        raise KernelError("paged_attention_maps: query rows are shorter than heads * maps * size")
+    if block_table.dim() != 2 or block_table.dtype != torch.int32 or block_table.stride(1) != 1:
+        raise KernelError("paged_attention_maps: block_table must be int32 [sequences, blocks]")
+    _i32(token_seq, "paged_attention_maps: token_seq", T)
+    _i32(positions, "paged_attention_maps: positions", T)
+    if differential is not None and maps != 2:
+        raise KernelError("paged_attention_maps: the differential combination needs two maps")
+    width = num_heads * (1 if differential is not None else maps) * dv
+    if out is None:
+        out = torch.empty((T, width), dtype=q.dtype, device=q.device)
+    if tuple(out.shape) != (T, width) or out.dtype != q.dtype:
+        raise KernelError("paged_attention_maps: bad output")
+    out_stride = _rows(out, "paged_attention_maps: out")
+    lam, eps, mult = differential if differential is not None else (0.0, 0.0, 1.0)
+    _lib.call("sa_paged_attention_maps", _ptr(q), _code(q), q_stride, _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
+              block_table.stride(0), _ptr(token_seq), _ptr(positions), _ptr(out), out_stride, T, num_heads, Kh, hd, dv,
+              page_size, int(window or 0), float(scale), int(maps), int(v_pages is None), int(differential is not None),
+              float(lam), float(eps), float(mult), _stream())
+    return out
+
+
 # --------------------------------------------------------------------------- norms behind parts, gates
 
 
@@ -756,6 +806,33 @@ def residual_add_norm(y: "torch.Tensor | PartialSums | None", residual: torch.Te
     _lib.call("sa_residual_add_norm", _ptr(y), _code(y) if y is not None else 0, ys, _ptr(weight),
               _code(weight) if weight is not None else 0, float(eps), int(plus_one), float(mult), _ptr(residual),
               _ptr(out), _code(out) if out is not None else 0, T, D, _stream())
+    return out
+
+
+def residual_add_next_norm(y: "torch.Tensor | PartialSums | None", residual: torch.Tensor, weight: torch.Tensor, *,
+                           eps: float, plus_one: bool = False, mult: float = 1.0,
+                           out_dtype: torch.dtype | None = None) -> torch.Tensor:
+    """residual += mult * y (y None: nothing is added); returns residual / sqrt(mean(residual^2) + eps) * (weight +
+    plus_one) in out_dtype: one pass over the rows."""
+    if isinstance(y, PartialSums):
+        y = y.materialize()
+    _dev(y, residual, weight)
+    T, D = residual.shape
+    if residual.dtype != torch.float32 or not residual.is_contiguous():
+        raise KernelError("residual_add_next_norm: the residual stream must be contiguous float32")
+    if weight.numel() != D or not weight.is_contiguous():
+        raise KernelError("residual_add_next_norm: the norm weight does not match the width")
+    ys = 0
+    if y is not None:
+        if tuple(y.shape) != (T, D):
+            raise KernelError(f"residual_add_next_norm: y {tuple(y.shape)} does not match the residual {T, D}")
+        ys = _rows(y, "residual_add_next_norm: y")
+    if D > 8192:
+        residual_add_norm(y, residual, mult=mult)
+        return rmsnorm(residual, weight, eps, plus_one, out_dtype or (y.dtype if y is not None else torch.float32))
+    out = torch.empty((T, D), dtype=out_dtype or (y.dtype if y is not None else torch.float32), device=residual.device)
+    _lib.call("sa_residual_add_next_norm", _ptr(y), _code(y) if y is not None else 0, ys, float(mult), _ptr(residual),
+              _ptr(weight), _code(weight), float(eps), int(plus_one), _ptr(out), _code(out), T, D, _stream())
     return out
 
 
@@ -845,6 +922,135 @@ def qk_norm_rope_cache_write(proj: torch.Tensor, positions: torch.Tensor, inv_fr
 
 
 # --------------------------------------------------------------------------- recurrent mixers
+
+
+def norm_rope_cache_write(proj: torch.Tensor, positions: torch.Tensor, freq: torch.Tensor | None, rot_dims: int,
+                          num_heads: int, num_kv_heads: int, key_dim: int, value_dim: int, *, rot_mult: float = 1.0,
+                          sub: int = 1, eps: float = 0.0, q_weight: torch.Tensor | None = None, q_norm_dims: int = 0,
+                          q_rot_at: int = 0, k_weight: torch.Tensor | None = None, k_norm_dims: int = 0,
+                          k_rot_at: int = 0, slot_mapping: torch.Tensor | None = None,
+                          k_pages: torch.Tensor | None = None, v_pages: torch.Tensor | None = None) -> torch.Tensor:
+    """In place on fused projection rows [H * dk | K * dk | K * dv | ...]: every query and key vector is `sub` equal
+    parts; in each part the first *_norm_dims entries are divided by their root mean square (eps inside the root) and
+    multiplied by *_weight (None: no norm), then the entries [*_rot_at, *_rot_at + rot_dims) turn in neighbouring pairs
+    (2p, 2p + 1) by position * freq[p], cos and sin times rot_mult.  Queries go back in place, keys into k_pages
+    [pages, K, P, dk], values (value_dim > 0) into v_pages [pages, K, dv, P]."""
+    _dev(proj, positions, freq, q_weight, k_weight, slot_mapping, k_pages, v_pages)
+    stride = _rows(proj, "norm_rope_cache_write: proj")
+    T = proj.shape[0]
+    H, K, dk, dv = int(num_heads), int(num_kv_heads), int(key_dim), int(value_dim)
+    if proj.shape[1] < (H + K) * dk + K * dv:
+        raise KernelError(f"norm_rope_cache_write: rows of {proj.shape[1]} are shorter than (H + K) dk + K dv")
+    _i32(positions, "norm_rope_cache_write: positions", T)
+    if rot_dims and (freq is None or freq.dtype != torch.float32 or freq.numel() != rot_dims // 2
+                     or not freq.is_contiguous() or rot_dims % 2):
+        raise KernelError("norm_rope_cache_write: freq must be float32 [rot_dims / 2], rot_dims even")
+    w_dtype = None
+    for w, n in ((q_weight, q_norm_dims), (k_weight, k_norm_dims)):
+        if w is not None:
+            if not w.is_contiguous() or w.numel() < n or (w_dtype is not None and w.dtype != w_dtype):
+                raise KernelError("norm_rope_cache_write: norm weights are contiguous, of one type, one entry per normed entry")
+            w_dtype = w.dtype
+    page_size = 1
+    if k_pages is not None:
+        if slot_mapping is None or (dv > 0 and v_pages is None):
+            raise KernelError("norm_rope_cache_write: key pages come with slots and, if there are values, value pages")
+        if k_pages.dim() != 4 or not k_pages.is_contiguous() or k_pages.dtype != proj.dtype \
+                or k_pages.shape[1] != K or k_pages.shape[3] != dk:
+            raise KernelError(f"norm_rope_cache_write: key pages {tuple(k_pages.shape)} do not match {K} heads of {dk}")
+        page_size = k_pages.shape[2]
+        if dv > 0 and (v_pages.dtype != proj.dtype or not v_pages.is_contiguous()
+                       or tuple(v_pages.shape) != (k_pages.shape[0], K, dv, page_size)):
+            raise KernelError(f"norm_rope_cache_write: value pages {tuple(v_pages.shape)} do not match")
+        if slot_mapping.dtype != torch.int64 or slot_mapping.numel() < T or not slot_mapping.is_contiguous():
+            raise KernelError("norm_rope_cache_write: slot_mapping must be int64 [T]")
+    _lib.call("sa_norm_rope_cache_write", _ptr(proj), _code(proj), stride, _ptr(positions), _ptr(freq), int(rot_dims),
+              float(rot_mult), _ptr(q_weight), int(q_norm_dims), int(q_rot_at), _ptr(k_weight), int(k_norm_dims),
+              int(k_rot_at), _CODES[w_dtype] if w_dtype is not None else 0, float(eps), int(sub), _ptr(slot_mapping),
+              _ptr(k_pages), _ptr(v_pages) if dv > 0 else None, T, H, K, dk, dv, int(page_size), _stream())
+    return proj
+
+
+def short_conv(x: torch.Tensor, taps: torch.Tensor, tails: torch.Tensor, seq_meta: torch.Tensor, num_seqs: int,
+               max_q_len: int, *, in_bias: torch.Tensor | None = None, out_bias: torch.Tensor | None = None,
+               silu: bool = False, update_tails: bool = True) -> torch.Tensor:
+    """`short_conv_silu` with the activation optional and two biases: y = act(sum_j taps[c, j] (x + in_bias)[t - ...]
+    + out_bias); the tails hold x + in_bias.  Returns float32 [T, C]."""
+    _dev(x, taps, tails, seq_meta, in_bias, out_bias)
+    stride = _rows(x, "short_conv: x")
+    T, C = x.shape
+    if taps.dim() != 2 or taps.shape[0] != C or not taps.is_contiguous():
+        raise KernelError(f"short_conv: taps {tuple(taps.shape)} for {C} channels")
+    n = taps.shape[1]
+    if tails.dtype != torch.float32 or tails.dim() != 2 or tails.stride(1) != 1 or tails.shape[1] < (n - 1) * C:
+        raise KernelError("short_conv: tails must be float32 [slots, >= (taps - 1) * channels]")
+    _seq_meta(seq_meta, num_seqs, "short_conv")
+    b_dtype = None
+    for b in (in_bias, out_bias):
+        if b is not None:
+            if b.numel() != C or not b.is_contiguous() or (b_dtype is not None and b.dtype != b_dtype):
+                raise KernelError("short_conv: biases are contiguous, of one type, one entry per channel")
+            b_dtype = b.dtype
+    out = torch.empty((T, C), dtype=torch.float32, device=x.device)
+    _lib.call("sa_short_conv", _ptr(x), _code(x), stride, _ptr(in_bias), _ptr(taps), _code(taps), n, _ptr(out_bias),
+              _CODES[b_dtype] if b_dtype is not None else 0, int(silu), _ptr(tails), tails.stride(0), _ptr(seq_meta),
+              int(num_seqs), int(max_q_len), _ptr(out), C, int(update_tails), _stream())
+    return out
+
+
+def head_product(x: torch.Tensor, w: torch.Tensor, *, in_stride: int | None = None, tail: int = 0,
+                 gate: torch.Tensor | None = None, out_dtype: torch.dtype | None = None) -> torch.Tensor:
+    """A product per head: out[t, h, :O] = w[h] x[t, h, :I] with w [H, O, I], summed in 32-bit.  x rows hold the
+    heads `in_stride` entries apart (default I + tail).  tail: the entries behind a head's inputs are copied behind its
+    outputs.  gate [T, H] (a view is fine): the outputs are multiplied by sigmoid(gate).  Returns [T, H * (O + tail)]."""
+    _dev(x, w, gate)
+    xs = _rows(x, "head_product: x")
+    T = x.shape[0]
+    if w.dim() != 3 or not w.is_contiguous():
+        raise KernelError("head_product: the weights are a contiguous [heads, outputs, inputs] tensor")
+    H, O, I = w.shape
+    hs = int(in_stride) if in_stride is not None else I + tail
+    if hs < I + tail or x.shape[1] < (H - 1) * hs + I + tail:
+        raise KernelError(f"head_product: rows of {x.shape[1]} do not hold {H} heads {hs} apart with {I + tail} entries")
+    gs = 0
+    if gate is not None:
+        gs = _rows(gate, "head_product: gate")
+        if gate.shape[0] != T or gate.shape[1] != H:
+            raise KernelError(f"head_product: gates {tuple(gate.shape)} are not [T, H]")
+    out = torch.empty((T, H * (O + tail)), dtype=out_dtype or x.dtype, device=x.device)
+    _lib.call("sa_head_product", _ptr(x), _code(x), xs, hs, _ptr(w), _code(w), _ptr(out), _code(out), out.stride(0),
+              O + tail, T, H, I, O, int(tail), _ptr(gate), _code(gate) if gate is not None else 0, gs, _stream())
+    return out
+
+
+def rglru_scan(u: torch.Tensor, gates: torch.Tensor, block: int, r_bias: torch.Tensor, i_bias: torch.Tensor,
+               lam: torch.Tensor, y: torch.Tensor, y_bias: torch.Tensor | None, state: torch.Tensor,
+               seq_meta: torch.Tensor, num_seqs: int, *, c: float = 8.0, out_dtype: torch.dtype | None = None) -> torch.Tensor:
+    """The real-gated linear recurrence, channel by channel over each request's tokens, from and into state [slots, C]
+    float32 (a view is fine): r = sigmoid(gr + r_bias), i = sigmoid(gi + i_bias), a = exp(-c r softplus(lam)),
+    S <- a S + sqrt(1 - a^2) i u; returns S * gelu_tanh(y + y_bias) in out_dtype.  u float32 [T, C]; gates float32
+    [T, 2 C], per block of `block` channels [gr | gi]; y [T, C] rows of the activation type."""
+    _dev(u, gates, r_bias, i_bias, lam, y, y_bias, state, seq_meta)
+    T, C = u.shape
+    if u.dtype != torch.float32 or not u.is_contiguous() or gates.dtype != torch.float32 or not gates.is_contiguous() \
+            or tuple(gates.shape) != (T, 2 * C):
+        raise KernelError("rglru_scan: u is contiguous float32 [T, C], gates contiguous float32 [T, 2 C]")
+    if block < 1 or C % block:
+        raise KernelError(f"rglru_scan: blocks of {block} do not divide {C} channels")
+    vecs = [r_bias, i_bias, lam] + ([y_bias] if y_bias is not None else [])
+    if any(v.numel() != C or not v.is_contiguous() or v.dtype != lam.dtype for v in vecs):
+        raise KernelError("rglru_scan: biases and lam are contiguous, of one type, one entry per channel")
+    ys = _rows(y, "rglru_scan: y")
+    if tuple(y.shape) != (T, C):
+        raise KernelError(f"rglru_scan: y {tuple(y.shape)} is not [T, C]")
+    if state.dtype != torch.float32 or state.dim() != 2 or state.stride(1) != 1 or state.shape[1] < C:
+        raise KernelError("rglru_scan: the state must be float32 [slots, >= channels]")
+    _seq_meta(seq_meta, num_seqs, "rglru_scan")
+    out = torch.empty((T, C), dtype=out_dtype or y.dtype, device=u.device)
+    _lib.call("sa_rglru_scan", _ptr(u), _ptr(gates), int(block), _ptr(r_bias), _ptr(i_bias), _ptr(lam), _code(lam),
+              float(c), _ptr(y), _code(y), ys, _ptr(y_bias), _ptr(state), state.stride(0), _ptr(seq_meta), int(num_seqs),
+              _ptr(out), _code(out), C, _stream())
+    return out
 
 
 def short_conv_silu(x: torch.Tensor, taps: torch.Tensor, tails: torch.Tensor, seq_meta: torch.Tensor, num_seqs: int,

@@ -215,3 +215,80 @@ class SinkAttention(Mixer):
         if self.bias:
             return ops.bias_add_(ops.gemm(o, self.o_proj), self.o_bias)
         return ops.gemm(o, self.o_proj, defer_sum=defer_sum)
+
+
+@MIXERS.register("differential_attention")
+class DifferentialAttention(Mixer):
+    """Grouped-query attention with two score maps per head over the same values.  A query row holds, head by head,
+    [map 1 | map 2] of `key_dim` entries each, a key row likewise per key head; every map of every head is divided by
+    its root mean square and multiplied by a weight of `key_dim` entries that all heads and maps share (`qk_norm`),
+    then its first entries are rotated (`position_encoding`: 'pair_rope').  With a_1, a_2 the maps' softmax results
+    over the window and lambda = exp(lq1 . lk1) - exp(lq2 . lk2) + diff (one number for the layer):
+
+        o = a_1 - lambda a_2;   o <- o / sqrt(mean(o^2) + norm_eps) * (1 - diff)   per head, over its values
+
+    q, k and v are one product; the cache holds key rows of 2 * key_dim entries and values of their own size."""
+
+    defers_sum = True
+
+    def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, key_dim: int, value_dim: int, scale: float,
+                 diff: float, norm_eps: float, qk_norm: bool = True, window: int | None = None,
+                 position_encoding: PartSpec | None = None):
+        if num_heads % num_kv_heads:
+            raise ValueError(f"differential_attention: {num_heads} heads do not split over {num_kv_heads} kv heads")
+        self.hidden_size, self.num_heads, self.num_kv_heads = int(hidden_size), int(num_heads), int(num_kv_heads)
+        self.key_dim, self.value_dim, self.scale = int(key_dim), int(value_dim), float(scale)
+        self.diff, self.norm_eps, self.qk_norm = float(diff), float(norm_eps), bool(qk_norm)
+        self.window = int(window) if window else None
+        self.position_encoding = (POSITION_ENCODINGS.build(position_encoding.kind, **position_encoding.params)
+                                  if position_encoding is not None else None)
+        if self.position_encoding is not None and not hasattr(self.position_encoding, "mult"):
+            raise ValueError("differential_attention: the position encoding must rotate neighbouring pairs (pair_rope)")
+        self.in_proj = self.o_proj = self.q_norm = self.k_norm = None
+        self.lam = 0.0
+
+    def param_specs(self):
+        D, H, K, dk, dv = self.hidden_size, self.num_heads, self.num_kv_heads, self.key_dim, self.value_dim
+        specs = {"q_proj": ParamSpec((H * 2 * dk, D)), "k_proj": ParamSpec((K * 2 * dk, D)),
+                 "v_proj": ParamSpec((K * dv, D)), "o_proj": ParamSpec((D, H * dv))}
+        if self.qk_norm:
+            specs.update(q_norm=ParamSpec((dk,), role="vector", init="norm"),
+                         k_norm=ParamSpec((dk,), role="vector", init="norm"))
+        for name in ("lq1", "lk1", "lq2", "lk2"):
+            specs[name] = ParamSpec((dk,), role="vector", init="norm")
+        return specs
+
+    def load(self, tensors):
+        t = tensors
+        self.in_proj = as_product_weight(torch.cat([t["q_proj"], t["k_proj"], t["v_proj"]], dim=0).contiguous())
+        self.o_proj = as_product_weight(t["o_proj"])
+        if self.qk_norm:
+            self.q_norm, self.k_norm = t["q_norm"].contiguous(), t["k_norm"].to(t["q_norm"].dtype).contiguous()
+        f = {n: t[n].to(torch.float32) for n in ("lq1", "lk1", "lq2", "lk2")}
+        # one number for the layer, in 32-bit
+        self.lam = float(torch.exp((f["lq1"] * f["lk1"]).sum()) - torch.exp((f["lq2"] * f["lk2"]).sum())
+                         + torch.tensor(self.diff, dtype=torch.float32))
+        if self.position_encoding is not None:
+            self.position_encoding.to_device(t["o_proj"].device)
+
+    def cache_need(self):
+        return PagedKVNeed(self.num_kv_heads, 2 * self.key_dim, self.window, self.value_dim)
+
+    def forward(self, x, ctx, cache, defer_sum=False):
+        H, K, dk, dv = self.num_heads, self.num_kv_heads, self.key_dim, self.value_dim
+        group = ctx.groups[cache.group_id]
+        proj = ops.gemm(x, self.in_proj)
+        pe = self.position_encoding
+        freq, rot_dims = pe.frequencies() if pe is not None else (None, 0)
+        write = cache.write
+        # every map of every head: norm, rotation; keys and values into their pages
+        ops.norm_rope_cache_write(proj, ctx.positions, freq, rot_dims, H, K, 2 * dk, dv,
+                                  rot_mult=pe.mult if pe is not None else 1.0, sub=2, eps=self.norm_eps,
+                                  q_weight=self.q_norm, q_norm_dims=dk if self.qk_norm else 0,
+                                  k_weight=self.k_norm, k_norm_dims=dk if self.qk_norm else 0,
+                                  slot_mapping=group.slot_mapping if write else None,
+                                  k_pages=cache.k_pages if write else None, v_pages=cache.v_pages if write else None)
+        o = ops.paged_attention_maps(proj, cache.k_pages, cache.v_pages, group.block_table, ctx.token_seq,
+                                     ctx.positions, H, scale=self.scale, maps=2, window=self.window,
+                                     differential=(self.lam, self.norm_eps, 1.0 - self.diff))
+        return ops.gemm(o, self.o_proj, defer_sum=defer_sum)

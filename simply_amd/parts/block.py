@@ -122,3 +122,43 @@ class PostNormBlock(Block):
         normed = n["post_mixer"].add_into(h, y, n["input"], ctx.dtype)
         y = self.feed_forward.forward(normed, ctx)
         return h, n["post_ffn"].add_into(h, y, next_norm, ctx.dtype)
+
+
+@BLOCKS.register("pre_norm")
+class PreNormBlock(Block):
+    """h += mult * mixer(pre_mixer(h));  h += mult * ffn(pre_ffn(h)): the parts read normed input, what they return is
+    added as it is, times a constant (`mult`, a residual multiplier).  A layer may have no feed-forward; then the
+    second step is left out.  Each sum runs in one kernel with the norm in front of the next part where that is an
+    RMSNorm."""
+
+    def __init__(self, mixer, feed_forward, norms, mult: float = 1.0):
+        super().__init__(mixer, feed_forward, norms)
+        self.mult = float(mult)
+        wanted = ("pre_mixer",) + (("pre_ffn",) if feed_forward is not None else ())
+        missing = [n for n in wanted if n not in self.norms]
+        if missing:
+            raise ValueError(f"pre_norm block: norms missing: {missing}")
+
+    def first_norm(self):
+        return self.norms["pre_mixer"]
+
+    def _add(self, h, y, norm, dtype):
+        """h += mult * y; returns norm(h), or None without a norm."""
+        if norm is not None and getattr(norm, "fusable_rms", False):
+            return ops.residual_add_next_norm(y, h, norm.scale, eps=norm.eps, plus_one=norm.scale_plus_one,
+                                              mult=self.mult, out_dtype=dtype)
+        ops.residual_add_norm(y, h, mult=self.mult)
+        return norm.forward(h, dtype) if norm is not None else None
+
+    def forward(self, h, ctx, cache, normed, next_norm):
+        n = self.norms
+        if isinstance(normed, PendingNorm):
+            normed, h = normed.materialize(), normed.residual
+        if normed is None:
+            normed = n["pre_mixer"].forward(h, ctx.dtype)
+        y = self.mixer.forward(normed, ctx, cache)
+        if self.feed_forward is None:
+            return h, self._add(h, y, next_norm, ctx.dtype)
+        normed = self._add(h, y, n["pre_ffn"], ctx.dtype)
+        y = self.feed_forward.forward(normed, ctx)
+        return h, self._add(h, y, next_norm, ctx.dtype)

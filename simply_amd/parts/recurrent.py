@@ -1,4 +1,6 @@
-"""A recurrent mixer: the gated delta rule.
+"""Recurrent mixers: the gated delta rule, and the real-gated linear recurrent unit (further down).
+
+The gated delta rule:
 
 Per head a matrix state S [key size, value size] in 32-bit, carried from token to token of a request:
 
@@ -71,4 +73,64 @@ class GatedDelta(Mixer):
         o = ops.delta_rule(qkv, gates, state, ctx.seq_meta, ctx.num_seqs, H, G, dk, dv)
         z = ops.gated_heads(o, proj[:, C:C + H * dv], H, dv, kind=ops.GATE_SILU, weight=self.norm, eps=self.norm_eps,
                             out_dtype=ctx.dtype)
+        return ops.gemm(z, self.o_proj)
+
+
+@MIXERS.register("rglru")
+class RGLRU(Mixer):
+    """A recurrent block with one number of state per channel.  Two branches of `width` channels from the mixer's
+    input: y = gelu_tanh(W_y h + b_y), and u = conv(W_x h + b_x), a causal convolution per channel (taps oldest first,
+    a bias behind it, no activation).  The channels are cut into `blocks` equal parts; in part b, with square matrices
+    R_b and I_b:
+
+        r = sigmoid(R_b u_b + b_r),  i = sigmoid(I_b u_b + b_i),  a = exp(-decay_mult r softplus(lam))
+        S <- a S + sqrt(1 - a^2) i u         (32-bit, from 0, no special case for a first token)
+
+    and the result is W_o (S * y).  The request's state is S and the convolution's last taps - 1 inputs, one float32
+    row of a state slot.  Gates, decays and the recurrence are 32-bit whatever the activation type is."""
+
+    def __init__(self, hidden_size: int, width: int, blocks: int, conv_taps: int, decay_mult: float = 8.0):
+        if blocks < 1 or width % blocks:
+            raise ValueError(f"rglru: {width} channels do not split into {blocks} equal parts")
+        if conv_taps < 1:
+            raise ValueError("rglru: the convolution has at least one tap")
+        self.hidden_size, self.width, self.blocks = int(hidden_size), int(width), int(blocks)
+        self.conv_taps, self.decay_mult = int(conv_taps), float(decay_mult)
+        self.block_size = self.width // self.blocks
+        self.in_proj = self.o_proj = self.gate_w = None
+
+    def param_specs(self):
+        D, C, B, n, bs = self.hidden_size, self.width, self.blocks, self.conv_taps, self.block_size
+        vec = dict(role="vector", init="norm")
+        return {"y_proj": ParamSpec((C, D)), "y_bias": ParamSpec((C,), **vec), "x_proj": ParamSpec((C, D)),
+                "x_bias": ParamSpec((C,), **vec), "conv": ParamSpec((C, n), role="vector"),
+                "conv_bias": ParamSpec((C,), **vec), "r_gate": ParamSpec((B, bs, bs)),
+                "r_bias": ParamSpec((B, bs), **vec), "i_gate": ParamSpec((B, bs, bs)), "i_bias": ParamSpec((B, bs), **vec),
+                "lam": ParamSpec((C,), **vec), "o_proj": ParamSpec((D, C))}
+
+    def load(self, tensors):
+        t = tensors
+        self.in_proj = as_product_weight(torch.cat([t["y_proj"], t["x_proj"]], dim=0).contiguous())   # rows [y | x]
+        self.o_proj = as_product_weight(t["o_proj"])
+        # per part the two gate matrices stacked: one product per part gives [r inputs | i inputs]
+        self.gate_w = torch.cat([t["r_gate"], t["i_gate"]], dim=1).contiguous()
+        vt = t["lam"].dtype
+        self.taps = t["conv"].contiguous()
+        for name in ("y_bias", "x_bias", "conv_bias", "r_bias", "i_bias", "lam"):
+            setattr(self, name, t[name].to(vt).reshape(-1).contiguous())
+
+    def cache_need(self):
+        return StateNeed((self.width * self.conv_taps,), torch.float32)   # S, then the convolution's taps - 1 inputs
+
+    def forward(self, x, ctx, cache):
+        if not cache.write:
+            raise RuntimeError("rglru: a recurrent state cannot be read through another entry's cache")
+        C = self.width
+        proj = ops.gemm(x, self.in_proj)
+        state, tails = cache.state[:, :C], cache.state[:, C:]
+        u = ops.short_conv(proj[:, C:2 * C], self.taps, tails, ctx.seq_meta, ctx.num_seqs, ctx.max_q_len,
+                           in_bias=self.x_bias, out_bias=self.conv_bias)
+        gates = ops.head_product(u, self.gate_w, out_dtype=torch.float32)
+        z = ops.rglru_scan(u, gates, self.block_size, self.r_bias, self.i_bias, self.lam, proj[:, :C], self.y_bias,
+                           state, ctx.seq_meta, ctx.num_seqs, c=self.decay_mult, out_dtype=ctx.dtype)
         return ops.gemm(z, self.o_proj)

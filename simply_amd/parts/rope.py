@@ -77,3 +77,80 @@ class PartialRoPE(PositionEncoding):
         inv_freq, dims = self.frequencies()
         # (the kernel's first H heads are rotated in place; no keys, no values, no norm)
         ops.qk_norm_rope_cache_write(x, positions, inv_freq, dims, None, num_heads, 0, head_dim, 1)
+
+
+@POSITION_ENCODINGS.register("pair_rope")
+class PairRoPE(PositionEncoding):
+    """Rotation of `dims` consecutive entries in neighbouring pairs (2i, 2i + 1): the pair (u, v) at position p
+    becomes mult * (u cos a - v sin a, v cos a + u sin a), a = p * f_i.  Where the rotated entries lie inside a
+    vector is the mixer's business.  The frequencies, from f_i = base^(-2i / dims):
+
+      scaling None                                   f_i, mult 1
+      {"kind": "linear", "factor"}                   f_i / factor, mult 1
+      {"kind": "ramp", "factor", "original", "fast", "slow"}
+          f_i / factor * r_i + f_i * (1 - r_i) with a ramp r_i over the pair index that runs from 0 to 1 between the
+          dimensions at which `fast` and `slow` turns fit into `original` positions, dim(t) = dims ln(original /
+          (2 pi t)) / (2 ln base): lo = max(floor(dim(fast)), 0), hi = min(ceil(dim(slow)), dims - 1),
+          r_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1); mult = 0.1 ln(factor) + 1 on cos and sin.
+
+    Frequencies are computed in float64 and rounded once to float32; the angle is their 32-bit product with the
+    position."""
+
+    def __init__(self, dims: int, base: float, scaling: "dict | None" = None):
+        if dims % 2 or dims < 0:
+            raise ValueError(f"pair_rope: {dims} rotated entries (an even number)")
+        if dims and base <= 0:
+            raise ValueError("pair_rope: the base must be positive")
+        self.dims, self.base = int(dims), float(base)
+        self.scaling = dict(scaling) if scaling else None
+        kind = self.scaling.get("kind") if self.scaling else None
+        if kind not in (None, "linear", "ramp"):
+            raise ValueError(f"pair_rope: unknown scaling {kind!r}; known: linear, ramp")
+        for key in (("factor",) if kind == "linear" else ("factor", "original", "fast", "slow") if kind else ()):
+            if not float(self.scaling.get(key, 0)) > 0:
+                raise ValueError(f"pair_rope: {kind} scaling needs a positive {key!r}")
+        self._freq: torch.Tensor | None = None
+
+    @property
+    def mult(self) -> float:
+        """The factor on cos and sin."""
+        import math
+
+        if self.scaling and self.scaling["kind"] == "ramp":
+            return 0.1 * math.log(float(self.scaling["factor"])) + 1.0
+        return 1.0
+
+    def freq_host(self) -> torch.Tensor:
+        import math
+
+        i = torch.arange(self.dims // 2, dtype=torch.float64)
+        f = self.base ** (-2.0 * i / max(self.dims, 1))
+        sc = self.scaling
+        if sc and sc["kind"] == "linear":
+            f = f / float(sc["factor"])
+        elif sc:
+            def dim_of(turns):
+                return self.dims * math.log(float(sc["original"]) / (2.0 * math.pi * float(turns))) / (2.0 * math.log(self.base))
+
+            lo = max(math.floor(dim_of(sc["fast"])), 0)
+            hi = min(math.ceil(dim_of(sc["slow"])), self.dims - 1)
+            ramp = torch.clamp((i - lo) / max(hi - lo, 0.001), 0.0, 1.0)
+            f = f / float(sc["factor"]) * ramp + f * (1.0 - ramp)
+        return f.to(torch.float32)
+
+    def to_device(self, device) -> None:
+        self._freq = self.freq_host().to(device)
+
+    def frequencies(self) -> tuple[torch.Tensor | None, int]:
+        """(float32 [dims / 2] on the device, dims): what the norm-and-rotate kernel of a mixer takes."""
+        if self.dims and self._freq is None:
+            raise RuntimeError("pair_rope: to_device() has not been called")
+        return (self._freq if self.dims else None), self.dims
+
+    def apply(self, x, positions, num_heads, head_dim, div=1.0):
+        if div != 1.0:
+            raise ValueError("pair_rope: no division")
+        freq, dims = self.frequencies()
+        if dims > head_dim:
+            raise ValueError(f"pair_rope: {dims} rotated entries in vectors of {head_dim}")
+        ops.norm_rope_cache_write(x, positions, freq, dims, num_heads, 0, head_dim, 0, rot_mult=self.mult)

@@ -604,3 +604,145 @@ def routed_experts(x, experts, weights, gate_w, up_w, down_w, activation, *, sha
         s = _f(shared)
         out = out + (s * torch.sigmoid(_f(shared_gate)[:, :1]) if shared_gate is not None else s)
     return out.to(out_dtype or x.dtype)
+
+
+# --------------------------------------------------------------------------- attention with several maps, latents, rglru
+
+
+def residual_add_next_norm(y, residual, weight, *, eps, plus_one=False, mult=1.0, out_dtype=None):
+    if hasattr(y, "materialize"):
+        y = y.materialize()
+    if y is not None:
+        residual.copy_((_f(residual) + mult * _f(y)).to(torch.float32))
+    h = _f(residual)
+    out = h / torch.sqrt((h * h).mean(-1, keepdim=True) + eps) * (_f(weight) + (1.0 if plus_one else 0.0))
+    return out.to(out_dtype or (y.dtype if y is not None else torch.float32))
+
+
+def paged_attention_maps(q, k_pages, v_pages, block_table, token_seq, positions, num_heads, *, scale, maps=1,
+                         value_dim=None, window=None, differential=None, out=None):
+    T = q.shape[0]
+    _, Kh, P, row = k_pages.shape
+    dk = row // maps
+    krows = stored_keys_as_rows(k_pages)
+    dv = v_pages.shape[2] if v_pages is not None else int(value_dim)
+    H = num_heads
+    G = H // Kh
+    width = H * (1 if differential is not None else maps) * dv
+    res = torch.empty((T, width), dtype=q.dtype, device=q.device)
+    for t in range(T):
+        pos = int(positions[t])
+        lo = max(pos - window + 1, 0) if window else 0
+        keys = torch.arange(lo, pos + 1, device=q.device)
+        pages = block_table[int(token_seq[t]), keys // P].long()
+        assert (pages >= 0).all(), "attention reads a key that has no page"
+        k = _f(krows[pages, :, keys % P]).reshape(len(keys), Kh, maps, dk)
+        v = _f(v_pages[pages, :, :, keys % P]) if v_pages is not None else _f(krows[pages, :, keys % P])[..., :dv]
+        qt = _f(q[t, :H * maps * dk]).reshape(Kh, G, maps, dk)
+        p = torch.softmax(torch.einsum("kgmd,nkmd->kgmn", qt, k) * scale, -1)
+        a = torch.einsum("kgmn,nkd->kgmd", p, v)            # [Kh, G, maps, dv]
+        if differential is not None:
+            lam, eps, mult = differential
+            o = a[:, :, 0] - lam * a[:, :, 1]
+            a = o / torch.sqrt((o * o).mean(-1, keepdim=True) + eps) * mult
+        res[t] = a.reshape(width).to(q.dtype)
+    if out is not None:
+        out.copy_(res)
+        return out
+    return res
+
+
+def norm_rope_cache_write(proj, positions, freq, rot_dims, num_heads, num_kv_heads, key_dim, value_dim, *, rot_mult=1.0,
+                          sub=1, eps=0.0, q_weight=None, q_norm_dims=0, q_rot_at=0, k_weight=None, k_norm_dims=0,
+                          k_rot_at=0, slot_mapping=None, k_pages=None, v_pages=None):
+    T = proj.shape[0]
+    H, K, dk, dv = num_heads, num_kv_heads, key_dim, value_dim
+    ds = dk // sub
+    ang = None
+    if rot_dims:
+        ang = positions.to(torch.float32)[:, None] * freq.to(torch.float32)[None, :]       # 32-bit angles
+        ang = ang.to(torch.float64 if PRECISE else torch.float32)[:, None, :]
+
+    def treat(x, weight, norm_dims, rot_at):    # x [T, n, ds]
+        x = x.clone()
+        if weight is not None and norm_dims:
+            part = x[..., :norm_dims]
+            x[..., :norm_dims] = part / torch.sqrt((part * part).mean(-1, keepdim=True) + eps) * _f(weight)[:norm_dims]
+        if rot_dims:
+            s, c = torch.sin(ang) * rot_mult, torch.cos(ang) * rot_mult
+            a = x[..., rot_at:rot_at + rot_dims:2].clone()
+            b = x[..., rot_at + 1:rot_at + rot_dims:2].clone()
+            x[..., rot_at:rot_at + rot_dims:2] = a * c - b * s
+            x[..., rot_at + 1:rot_at + rot_dims:2] = b * c + a * s
+        return x
+
+    if H:
+        q = treat(_f(proj[:, :H * dk]).reshape(T, H * sub, ds), q_weight, q_norm_dims, q_rot_at)
+        proj[:, :H * dk] = q.reshape(T, H * dk).to(proj.dtype)
+    if k_pages is None or K == 0:
+        return proj
+    k = treat(_f(proj[:, H * dk:(H + K) * dk]).reshape(T, K * sub, ds), k_weight, k_norm_dims, k_rot_at)
+    P = k_pages.shape[2]
+    page, off = (slot_mapping[:T] // P).long(), (slot_mapping[:T] % P).long()
+    krows = stored_keys_as_rows(k_pages)
+    krows[page, :, off] = k.reshape(T, K, dk).to(k_pages.dtype)
+    k_pages.copy_(rows_as_stored_keys(krows))
+    if dv:
+        v = proj[:, (H + K) * dk:(H + K) * dk + K * dv]
+        v_pages[page, :, :, off] = v.reshape(T, K, dv).to(v_pages.dtype)
+    return proj
+
+
+def short_conv(x, taps, tails, seq_meta, num_seqs, max_q_len, *, in_bias=None, out_bias=None, silu=False,
+               update_tails=True):
+    T, C = x.shape
+    n = taps.shape[1]
+    y = torch.empty((T, C), dtype=torch.float32, device=x.device)
+    w = _f(taps)
+    for slot, first, count, _ in seq_meta[:num_seqs].tolist():
+        old = _f(tails[slot, :(n - 1) * C]).reshape(n - 1, C)
+        new = _f(x[first:first + count])
+        if in_bias is not None:
+            new = new + _f(in_bias)[None, :]
+        xs = torch.cat([old, new], dim=0)
+        acc = sum(xs[j:j + count] * w[:, j][None, :] for j in range(n))
+        if out_bias is not None:
+            acc = acc + _f(out_bias)[None, :]
+        y[first:first + count] = (acc * torch.sigmoid(acc) if silu else acc).to(torch.float32)
+        if update_tails and n > 1:
+            tails[slot, :(n - 1) * C] = xs[count:].reshape(-1).to(torch.float32)
+    return y
+
+
+def head_product(x, w, *, in_stride=None, tail=0, gate=None, out_dtype=None):
+    T = x.shape[0]
+    H, O, I = w.shape
+    hs = in_stride if in_stride is not None else I + tail
+    xf = _f(x)
+    heads = torch.stack([xf[:, h * hs:h * hs + I + tail] for h in range(H)], dim=1)       # [T, H, I + tail]
+    o = torch.einsum("thi,hoi->tho", heads[..., :I], _f(w))
+    if gate is not None:
+        o = o * torch.sigmoid(_f(gate))[:, :, None]
+    return torch.cat([o, heads[..., I:]], dim=-1).reshape(T, H * (O + tail)).to(out_dtype or x.dtype)
+
+
+def rglru_scan(u, gates, block, r_bias, i_bias, lam, y, y_bias, state, seq_meta, num_seqs, *, c=8.0, out_dtype=None):
+    T, C = u.shape
+    g = _f(gates).reshape(T, C // block, 2, block)
+    r = torch.sigmoid(g[:, :, 0].reshape(T, C) + _f(r_bias))
+    i = torch.sigmoid(g[:, :, 1].reshape(T, C) + _f(i_bias))
+    lm = _f(lam)
+    sp = torch.where(lm > 30.0, lm, torch.log1p(torch.exp(torch.clamp(lm, max=30.0))))
+    log_a = -c * r * sp
+    a, m = torch.exp(log_a), torch.sqrt(-torch.expm1(2.0 * log_a))
+    z = _f(y) + (_f(y_bias) if y_bias is not None else 0.0)
+    gy = gelu_tanh(z)
+    uf = _f(u)
+    out = torch.empty((T, C), dtype=out_dtype or y.dtype, device=u.device)
+    for slot, first, count, _ in seq_meta[:num_seqs].tolist():
+        S = _f(state[slot, :C])
+        for t in range(first, first + count):
+            S = a[t] * S + m[t] * (i[t] * uf[t])
+            out[t] = (S * gy[t]).to(out.dtype)
+        state[slot, :C] = S.to(torch.float32)
+    return out
