@@ -253,3 +253,11 @@ def forward(w, cfg, tokens, dtype=torch.float64, layers_out: list | None = None)
     logits = rms_norm(x, w["final.norm"].to(dtype), eps) @ w["head"].to(dtype).T
     cap = cfg.get("logit_softcap")
     return cap * torch.tanh(logits / cap) if cap else logits
+
+
+def greedy(w, cfg, prompt, steps: int, dtype=torch.float64) -> list[int]:
+    """`steps` tokens after `prompt`, each the largest logit's, the whole sequence run anew every time."""
+    tokens = list(prompt)
+    for _ in range(steps):
+        tokens.append(int(forward(w, cfg, tokens, dtype)[-1].argmax()))
+    return tokens[len(prompt):]
