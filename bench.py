@@ -499,6 +499,59 @@ def run_nemidra(args):
             torch.cuda.empty_cache()
 
 
+# --only tabupel: layer sizes that resemble a real model's, for the Tabupel design (two recurrent layers, one with
+# differential attention behind a window, one with latent attention, in turn; a gated feed-forward of as many parameters
+# as Zenuzen's dense one in every layer) and, beside it, the closest model that the engine has, Zenuzen, at equal
+# width, depth, heads and head size
+def tabupel_config(size: dict, layers: int) -> dict:
+    W, H, K, d = size["width"], size["heads"], size["kv_heads"], size["dim"]
+    ff = (2 * size["ff"] // 3 + 255) // 256 * 256    # three matrices instead of two
+    out = []
+    for i in range(layers):
+        mlp = {"kind": "dense", "ff": ff}
+        if i % 4 == 2:
+            out.append({"type": "attention", "mlp": mlp,
+                        "mixer": {"heads": H, "kv_heads": K, "dim": d // 2, "vdim": d, "scale": (d // 2) ** -0.5, "diff": 0.3,
+                                  "mask": {"size": 1024},
+                                  "rot": {"dims": d // 4, "base": 1000000.0, "scaling": {"factor": 8.0}}}})
+        elif i % 4 == 3:
+            out.append({"type": "latent_attention", "mlp": mlp,
+                        "mixer": {"heads": H, "dim": d, "rot_dim": 64, "vdim": d, "q_rank": 3 * W // 4, "kv_rank": 512,
+                                  "scale": (d + 64) ** -0.5,
+                                  "rot": {"dims": 64, "base": 20000.0,
+                                          "scaling": {"factor": 2.0, "original": 2048, "fast": 32.0, "slow": 1.0}}}})
+        else:
+            out.append({"type": "rglru", "mlp": mlp, "mixer": {"width": W, "blocks": H, "conv": 4}})
+    return {"architecture": "Tabupel", "vocab": size["vocab"], "width": W, "residual_mult": 0.7, "norm": {"eps": 1e-5},
+            "layers": out, "logit_softcap": 15.0}
+
+
+def run_tabupel(args):
+    import torch
+    from simply_amd.config import config_from_dict
+    from simply_amd.engine.loading import random_model
+
+    tdtype = torch.bfloat16 if args.dtype == "bfloat16" else torch.float32
+    layers = args.layers or 8
+    for name in args.sizes.split(","):
+        size = ZENUZEN_SIZES[name]
+        for label, d in (("tabupel", tabupel_config(size, layers)), ("zenuzen-equal-size", zenuzen_config(size, layers))):
+            if args.alone and label != "tabupel":
+                continue
+            cfg = config_from_dict(d)
+            model = random_model(cfg, 0, tdtype, torch.device("cuda:0"), std=0.02)
+            pt, dt = run_executor_bench(model, size["vocab"], args.prefill_tokens, args.batch, args.context, args.steps,
+                                        args.warmup, args.page_size, args.dtype)
+            print(json.dumps({"metric": "prefill and decode tokens/s through the step function", "model": label,
+                              "size": name, "width": size["width"], "layers": layers,
+                              "prefill_tokens": args.prefill_tokens, "prefill_tokens_per_s": round(args.prefill_tokens / pt, 1),
+                              "prefill_ms": round(pt * 1e3, 3), "batch": args.batch, "context": args.context,
+                              "decode_tokens_per_s": round(args.batch / dt, 1), "decode_ms_per_step": round(dt * 1e3, 3),
+                              "dtype": args.dtype, "data": "synthetic"}), flush=True)
+            del model
+            torch.cuda.empty_cache()
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -514,7 +567,7 @@ def main():
     ap.add_argument("--batches", default="1,8,32,64", help="--only decode-grid: the batch sizes")
     ap.add_argument("--contexts", default="1024,4096,8192", help="--only decode-grid: the context lengths")
     ap.add_argument("--only", default="all", choices=["all", "decode", "decode-grid", "prefill", "prefill-chunked", "products",
-                                                      "gated-products", "ceilings", "zenuzen", "nemidra"],
+                                                      "gated-products", "ceilings", "zenuzen", "nemidra", "tabupel"],
                     help="measure one part alone (for profiles); the line then holds that part only.  products / "
                          "gated-products: the sweep of the product kernels over rows and weight sizes; ceilings: "
                          "what the GPU itself reaches in reading HBM and in bfloat16 MFMA instructions")
@@ -522,8 +575,8 @@ def main():
                     help="decode steps run one at a time after the timed ones, for the p50 and p99 of a step's latency")
     ap.add_argument("--shape", default="2b", choices=sorted(SHAPES), help="layer sizes: Gemma 2 2B (the default), 9B, 27B")
     ap.add_argument("--sizes", default="small,medium,large",
-                    help="--only zenuzen / nemidra: which of the layer sizes small, medium, large (8 layers each, or --layers)")
-    ap.add_argument("--alone", action="store_true", help="--only nemidra: without the closest model beside it (for profiles)")
+                    help="--only zenuzen / nemidra / tabupel: which of the layer sizes small, medium, large (8 layers each, or --layers)")
+    ap.add_argument("--alone", action="store_true", help="--only nemidra / tabupel: without the closest model beside it (for profiles)")
     ap.add_argument("--requests", type=int, default=0,
                     help="instead of timed decode steps: a workload of this many requests through the scheduler")
     ap.add_argument("--prompt-min", type=int, default=128)
@@ -552,6 +605,9 @@ def main():
         return
     if args.only == "nemidra":
         run_nemidra(args)
+        return
+    if args.only == "tabupel":
+        run_tabupel(args)
         return
     d = dict(GEMMA2_2B, **SHAPES[args.shape])
     full_layers = d["num_hidden_layers"]

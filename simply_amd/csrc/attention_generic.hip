@@ -44,7 +44,11 @@ __global__ __launch_bounds__(kThreads) void paged_attention_generic_kernel(
     const int* __restrict__ block_table, int table_stride, const int* __restrict__ token_seq,
     const int* __restrict__ positions, T* __restrict__ out, int64_t out_stride, int Kh, int G, int hd, int hd_v,
     int page_size, int window, float soft_cap, float scale, const void* __restrict__ sinks, int sinks_dtype,
-    AttentionOptions opt) {
+    AttentionOptions opt, int G_all) {
+  // G_all query vectors per key/value head, of which this workgroup takes G (the last one of a head what is left):
+  // many heads over one key head need not fit into one workgroup's LDS
+  const int gz = blockIdx.z * G;          // the workgroup's first vector among its key head's
+  if (G > G_all - gz) G = G_all - gz;
   extern __shared__ float smem[];
   __shared__ float red_s[16];
   float* q_s = smem;                      // [G][hd]
@@ -65,7 +69,7 @@ __global__ __launch_bounds__(kThreads) void paged_attention_generic_kernel(
 
   for (int i = tid; i < G * hd; i += kThreads) {
     const int g = i / hd, d = i % hd;
-    q_s[i] = to_float(q[static_cast<size_t>(t) * q_stride + static_cast<size_t>(kh * G + g) * hd + d]);
+    q_s[i] = to_float(q[static_cast<size_t>(t) * q_stride + static_cast<size_t>(kh * G_all + gz + g) * hd + d]);
   }
   for (int g = tid; g < G; g += kThreads) {
     m_s[g] = -INFINITY;
@@ -191,7 +195,7 @@ __global__ __launch_bounds__(kThreads) void paged_attention_generic_kernel(
         for (int s = 0; s < kMaxDimsPerThread; ++s) {
           const int d = tid + s * kThreads;
           if (d < hd_v)
-            out[static_cast<size_t>(t) * out_stride + static_cast<size_t>((kh * G + g0) / 2 + p) * hd_v + d] =
+            out[static_cast<size_t>(t) * out_stride + static_cast<size_t>((kh * G_all + gz + g0) / 2 + p) * hd_v + d] =
                 from_float<T>(o[s][p] * r);
         }
       }
@@ -206,8 +210,8 @@ __global__ __launch_bounds__(kThreads) void paged_attention_generic_kernel(
           if (g < gn) {
             // a sink is one more term of the softmax's sum, exp(sink - maximum), without a value
             float l = l_s[g0 + g];
-            if (sinks != nullptr) l += expf(load_f(sinks, sinks_dtype, kh * G + g0 + g) - m_s[g0 + g]);
-            out[static_cast<size_t>(t) * out_stride + static_cast<size_t>(kh * G + g0 + g) * hd_v + d] =
+            if (sinks != nullptr) l += expf(load_f(sinks, sinks_dtype, kh * G_all + gz + g0 + g) - m_s[g0 + g]);
+            out[static_cast<size_t>(t) * out_stride + static_cast<size_t>(kh * G_all + gz + g0 + g) * hd_v + d] =
                 from_float<T>(acc[s][g] / l);
           }
       }
@@ -220,18 +224,18 @@ static void launch_generic(const void* q, int dtype, int64_t q_stride, const voi
                            const int* block_table, int table_stride, const int* token_seq, const int* positions,
                            void* out, int64_t out_stride, int T, int Kh, int G, int hd, int hd_v, int page_size,
                            int window, float soft_cap, float scale, const void* sinks, int sinks_dtype,
-                           AttentionOptions opt, size_t smem, hipStream_t stream) {
-  const dim3 grid(T, Kh);
+                           AttentionOptions opt, size_t smem, int G_all, hipStream_t stream) {
+  const dim3 grid(T, Kh, (G_all + G - 1) / G);
   if (dtype == kF32)
     paged_attention_generic_kernel<float, M><<<grid, kThreads, smem, stream>>>(
         static_cast<const float*>(q), q_stride, static_cast<const float*>(k_pages),
         static_cast<const float*>(v_pages), block_table, table_stride, token_seq, positions, static_cast<float*>(out),
-        out_stride, Kh, G, hd, hd_v, page_size, window, soft_cap, scale, sinks, sinks_dtype, opt);
+        out_stride, Kh, G, hd, hd_v, page_size, window, soft_cap, scale, sinks, sinks_dtype, opt, G_all);
   else
     paged_attention_generic_kernel<bf16, M><<<grid, kThreads, smem, stream>>>(
         static_cast<const bf16*>(q), q_stride, static_cast<const bf16*>(k_pages), static_cast<const bf16*>(v_pages),
         block_table, table_stride, token_seq, positions, static_cast<bf16*>(out), out_stride, Kh, G, hd, hd_v, page_size,
-        window, soft_cap, scale, sinks, sinks_dtype, opt);
+        window, soft_cap, scale, sinks, sinks_dtype, opt, G_all);
 }
 
 int paged_attention_generic(const void* q, int dtype, int64_t q_stride, const void* k_pages, const void* v_pages,
@@ -240,7 +244,7 @@ int paged_attention_generic(const void* q, int dtype, int64_t q_stride, const vo
                             float soft_cap, hipStream_t stream, int hd_v, float scale, const void* sinks,
                             int sinks_dtype, int maps, int values_in_keys, int differential, float lambda, float eps,
                             float mult) {
-  const int G = H / Kh * maps;   // query vectors per key/value head
+  int G = H / Kh * maps;   // query vectors per key/value head (below: per workgroup)
   if (hd_v <= 0) hd_v = hd;
   if (maps != 1 && maps != 2) {
     set_error("paged_attention: %d score maps per head (1 or 2)", maps);
@@ -262,11 +266,16 @@ int paged_attention_generic(const void* q, int dtype, int64_t q_stride, const vo
     set_error("paged_attention: value size %d is above the largest supported (%d)", hd_v, kThreads * kMaxDimsPerThread);
     return 1;
   }
-  const size_t smem = sizeof(float) * (static_cast<size_t>(G) * hd + static_cast<size_t>(G) * kChunk + 3 * G) +
-                      sizeof(int) * kChunk;
+  // the query vectors of a key head are cut over workgroups (in multiples of 8, the heads that run side by side) until
+  // a workgroup's share fits into LDS
+  const int G_all = G;
+  auto lds = [&](int g) {
+    return sizeof(float) * (static_cast<size_t>(g) * hd + static_cast<size_t>(g) * kChunk + 3 * g) + sizeof(int) * kChunk;
+  };
+  while (lds(G) > 64 * 1024 && G > 8) G = ((G + 1) / 2 + 7) / 8 * 8;
+  const size_t smem = lds(G);
   if (smem > 64 * 1024) {
-    set_error("paged_attention: %d query vectors per key head of size %d need %zu bytes of LDS (limit 65536)", G,
-              hd, smem);
+    set_error("paged_attention: %d query vectors of size %d need %zu bytes of LDS (limit 65536)", G, hd, smem);
     return 1;
   }
   AttentionOptions opt;
@@ -278,11 +287,11 @@ int paged_attention_generic(const void* q, int dtype, int64_t q_stride, const vo
   if (maps == 2)
     launch_generic<2>(q, dtype, q_stride, k_pages, v_pages, block_table, table_stride, token_seq, positions, out,
                       out_stride, T, Kh, G, hd, hd_v, page_size, window, soft_cap, scale, sinks, sinks_dtype, opt, smem,
-                      stream);
+                      G_all, stream);
   else
     launch_generic<1>(q, dtype, q_stride, k_pages, v_pages, block_table, table_stride, token_seq, positions, out,
                       out_stride, T, Kh, G, hd, hd_v, page_size, window, soft_cap, scale, sinks, sinks_dtype, opt, smem,
-                      stream);
+                      G_all, stream);
   return check_launch("paged_attention_generic");
 }
 

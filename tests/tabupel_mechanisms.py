@@ -359,14 +359,16 @@ def differential_part(device, dtype, sizes=(40, 6, 2, 10, 14), window=9, page_si
         close(got, want, 2e-5 if dtype == torch.float32 else 6e-2, f"cuts {c[:4]}")
 
 
-def latent_part(device, dtype, sizes=(40, 3, 12, 8, 10, 20, 24), window=13, page_size=4, length=61, cuts=CUTS):
+def latent_part(device, dtype, sizes=(40, 3, 12, 8, 10, 20, 24), window=13, page_size=4, length=61, cuts=CUTS, std=0.3):
+    """std: of the matrices (wide layers want smaller ones, or the scores grow so large that a bfloat16 run's rounding,
+    the plain implementation's own with roundings at the same places included, moves whole softmax sums)."""
     D, H, dk, dr, dv, Rq, R = sizes
     sc = {"factor": 3.0, "original": 64, "fast": 8.0, "slow": 1.0}
     m = {"heads": H, "dim": dk, "rot_dim": dr, "vdim": dv, "q_rank": Rq, "kv_rank": R, "scale": 0.3,
          "mask": {"size": window}, "rot": {"dims": dr, "base": 1000.0, "scaling": sc}}
-    p = {"dq": rand((Rq, D), 70, 0.3), "dq.norm": rand((Rq,), 71), "uq": rand((H * (dk + dr), Rq), 72, 0.3),
-         "dkv": rand((R + dr, D), 73, 0.3), "dkv.norm": rand((R,), 74), "uk": rand((H * dk, R), 75, 0.3),
-         "uv": rand((H * dv, R), 76, 0.3), "g": rand((H, D), 77, 0.3), "o": rand((D, H * dv), 78, 0.3)}
+    p = {"dq": rand((Rq, D), 70, std), "dq.norm": rand((Rq,), 71), "uq": rand((H * (dk + dr), Rq), 72, std),
+         "dkv": rand((R + dr, D), 73, std), "dkv.norm": rand((R,), 74), "uk": rand((H * dk, R), 75, std),
+         "uv": rand((H * dv, R), 76, std), "g": rand((H, D), 77, std), "o": rand((D, H * dv), 78, std)}
     p = {n: t.to(dtype).double() for n, t in p.items()}
     x = rand((length, D), 79).to(dtype)
     want = plain.latent_attention(x.double(), p, m, 1e-5)

@@ -40,6 +40,12 @@ def test_kernels_on_pages_of_sixteen_keys():
         mech.latent_attention_edges(ops, DEV, dtype, page_size=16, sizes=(3, 24, 8))
 
 
+def test_many_heads_over_one_key_head():
+    """More query vectors over one key head than a workgroup's LDS holds: the heads are cut over workgroups."""
+    mech.latent_attention_edges(ops, DEV, torch.bfloat16, page_size=16, sizes=(40, 416, 32))
+    mech.differential_attention_edges(ops, DEV, torch.float32, page_size=16, sizes=(18, 1, 512, 40))
+
+
 def test_recurrence_in_portions_and_other_taps():
     mech.recurrence(ops, DEV, torch.float32, cuts=(1, 2, 40, 1, 46))
     mech.recurrence(ops, DEV, torch.bfloat16, T=400, cuts=(100, 1, 129, 64, 2, 104), block=16)
@@ -69,7 +75,7 @@ def test_parts_at_aligned_sizes():
     cuts = ([300], [268] + [1] * 32, [17] * 17 + [11])
     mech.differential_part(DEV, torch.bfloat16, sizes=(128, 4, 2, 64, 128), window=48, page_size=16, length=300, cuts=cuts)
     mech.latent_part(DEV, torch.bfloat16, sizes=(128, 4, 64, 32, 64, 96, 128), window=80, page_size=16, length=300,
-                     cuts=cuts)
+                     cuts=cuts, std=0.1)
     mech.rglru_part(DEV, torch.bfloat16, sizes=(128, 128, 2, 4), length=300, cuts=cuts)
 
 
