@@ -297,6 +297,17 @@ int sa_paged_attention_maps(const void* q, int dtype, int64_t q_stride, const vo
                             int window, float scale, int maps, int values_in_keys, int differential, float lambda,
                             float eps, float mult, hipStream_t stream);
 
+// sa_paged_attention_maps in bfloat16 on the matrix cores, over units of few rows (csrc/attention_maps.hip).
+int sa_attention_maps_heads_per_unit(int H, int Kh);
+int sa_paged_attention_maps_units_takes(int H, int Kh, int maps, int hd, int hd_v, int page_size, int64_t q_stride,
+                                        const void* q);
+int sa_paged_attention_maps_units(const void* q, int64_t q_stride, const void* k_pages, const void* v_pages,
+                                  const int* block_table, int table_stride, const int* units, int unit_begin,
+                                  int unit_count, void* out, int64_t out_stride, int H, int Kh, int hd, int hd_v,
+                                  int page_size, int window, float scale, int maps, int differential, float lambda,
+                                  float eps, float mult, int max_kv_len, int max_q_len, void* workspace,
+                                  size_t workspace_bytes, hipStream_t stream);
+
 // residual += mult * norm(y; w) (w null: + mult * y; y null: nothing is added), then, if out is not null, out = the
 // residual in out's type: the sum of a block that norms what a part returns, and the hand-over to a next part that
 // has no norm in front of it.  The norm is y / sqrt(mean(y^2) + eps) * (w + plus_one).
@@ -334,12 +345,13 @@ int sa_residual_add_next_norm(const void* y, int y_dtype, int64_t y_stride, floa
 // multiplied by *_weight [>= *_norm_dims] (null: no norm), then the entries [*_rot_at, *_rot_at + rot_dims) turn in
 // neighbouring pairs (2p, 2p + 1) by position * freq[p], cos and sin times rot_mult.  Queries go back in place, keys
 // into key pages [num_pages, K, page_size, dk], values (dv > 0) into value pages [num_pages, K, dv, page_size].
-// k_pages null: nothing is written (then K is best 0).
+// k_pages null: nothing is written (then K is best 0).  key_values > 0 (with dv == 0): the first key_values entries of
+// every key row, as stored, also go into value pages [num_pages, K, key_values, page_size].
 int sa_norm_rope_cache_write(void* proj, int dtype, int64_t row_stride, const int* positions, const float* freq,
                              int rot_dims, float rot_mult, const void* q_weight, int q_norm_dims, int q_rot_at,
                              const void* k_weight, int k_norm_dims, int k_rot_at, int w_dtype, float eps, int sub,
                              const int64_t* slot_mapping, void* k_pages, void* v_pages, int T, int H, int K, int dk,
-                             int dv, int page_size, hipStream_t stream);
+                             int dv, int page_size, int key_values, hipStream_t stream);
 
 // y[t, c] = act(sum_j taps[c, j] (x[t - (n - 1 - j), c] + in_bias[c]) + out_bias[c]), act silu or none, as
 // sa_short_conv_silu below; either bias may be null; the tails hold x + in_bias.  Biases are of bias_dtype.

@@ -283,7 +283,9 @@ __global__ __launch_bounds__(kWave) void norm_rope_cache_write_kernel(
     T* __restrict__ proj, int64_t row_stride, const int* __restrict__ positions, const float* __restrict__ freq,
     int rot_dims, float rot_mult, HeadNormRope qn, HeadNormRope kn, int w_dtype, float eps, int sub,
     const int64_t* __restrict__ slot_mapping, T* __restrict__ k_pages, T* __restrict__ v_pages, int H, int K, int dk,
-    int dv, int page_size) {
+    int dv, int page_size, int key_values) {
+  // key_values > 0: a key row's first key_values entries, as they are stored, are the token's values as well (a latent
+  // that is scored and read): they also go into value pages [num_pages, K, key_values, page_size]
   const int t = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
   T* row = proj + static_cast<size_t>(t) * row_stride;
   if (head < H + K) {
@@ -341,8 +343,14 @@ __global__ __launch_bounds__(kWave) void norm_rope_cache_write_kernel(
           cs *= rot_mult;
           v = (e & 1) == 0 ? v * cs - o * sn : v * cs + o * sn;
         }
-        if (is_q) src[i] = from_float<T>(v);
-        else dst[key_index(tiled, page_size, dk, koff, part * ds + i)] = from_float<T>(v);
+        if (is_q) {
+          src[i] = from_float<T>(v);
+        } else {
+          dst[key_index(tiled, page_size, dk, koff, part * ds + i)] = from_float<T>(v);
+          if (part * ds + i < key_values)
+            v_pages[(((slot / page_size) * K + (head - H)) * key_values + part * ds + i) * page_size + koff] =
+                from_float<T>(v);
+        }
       }
     }
     return;
@@ -481,8 +489,11 @@ extern "C" int sa_norm_rope_cache_write(void* proj, int dtype, int64_t row_strid
                                         int q_norm_dims, int q_rot_at, const void* k_weight, int k_norm_dims,
                                         int k_rot_at, int w_dtype, float eps, int sub, const int64_t* slot_mapping,
                                         void* k_pages, void* v_pages, int T, int H, int K, int dk, int dv,
-                                        int page_size, hipStream_t stream) {
+                                        int page_size, int key_values, hipStream_t stream) {
   if (T == 0) return 0;
+  SA_REQUIRE(key_values >= 0 && key_values <= dk && (key_values == 0 || (dv == 0 && v_pages != nullptr)),
+             "norm_rope_cache_write: %d of a key row's %d entries as values (then there are value pages and no values "
+             "of their own)", key_values, dk);
   SA_REQUIRE(T > 0 && H >= 0 && K >= 0 && H + K > 0 && dk > 0 && dv >= 0 && page_size > 0 && sub > 0,
              "norm_rope_cache_write: bad sizes T=%d H=%d K=%d dk=%d dv=%d P=%d sub=%d", T, H, K, dk, dv, page_size, sub);
   SA_REQUIRE(dk % sub == 0 && dk / sub <= kPartPerLane * kWave,
@@ -504,11 +515,11 @@ extern "C" int sa_norm_rope_cache_write(void* proj, int dtype, int64_t row_strid
   if (dtype == kF32)
     norm_rope_cache_write_kernel<float><<<grid, kWave, 0, stream>>>(
         static_cast<float*>(proj), row_stride, positions, freq, rot_dims, rot_mult, qn, kn, w_dtype, eps, sub,
-        slot_mapping, static_cast<float*>(k_pages), static_cast<float*>(v_pages), H, K, dk, dv, page_size);
+        slot_mapping, static_cast<float*>(k_pages), static_cast<float*>(v_pages), H, K, dk, dv, page_size, key_values);
   else if (dtype == kBF16)
     norm_rope_cache_write_kernel<bf16><<<grid, kWave, 0, stream>>>(
         static_cast<bf16*>(proj), row_stride, positions, freq, rot_dims, rot_mult, qn, kn, w_dtype, eps, sub,
-        slot_mapping, static_cast<bf16*>(k_pages), static_cast<bf16*>(v_pages), H, K, dk, dv, page_size);
+        slot_mapping, static_cast<bf16*>(k_pages), static_cast<bf16*>(v_pages), H, K, dk, dv, page_size, key_values);
   else
     SA_REQUIRE(false, "norm_rope_cache_write: unknown dtype %d", dtype);
   return check_launch("norm_rope_cache_write");

@@ -67,7 +67,11 @@ _SIGNATURES = {
     "sa_paged_attention_maps": [_P, _I, _L, _P, _P, _P, _I, _P, _P, _P, _L, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _F,
                                 _F, _F, _P],
     "sa_norm_rope_cache_write": [_P, _I, _L, _P, _P, _I, _F, _P, _I, _I, _P, _I, _I, _I, _F, _I, _P, _P, _P, _I, _I, _I,
-                                 _I, _I, _I, _P],
+                                 _I, _I, _I, _I, _P],
+    "sa_attention_maps_heads_per_unit": [_I, _I],
+    "sa_paged_attention_maps_units_takes": [_I, _I, _I, _I, _I, _I, _L, _P],
+    "sa_paged_attention_maps_units": [_P, _L, _P, _P, _P, _I, _P, _I, _I, _P, _L, _I, _I, _I, _I, _I, _I, _F, _I, _I, _F,
+                                      _F, _F, _I, _I, _P, _L, _P],
     "sa_residual_add_next_norm": [_P, _I, _L, _F, _P, _P, _I, _F, _I, _P, _I, _I, _I, _P],
     "sa_short_conv": [_P, _I, _L, _P, _P, _I, _I, _P, _I, _I, _P, _L, _P, _I, _I, _P, _I, _I, _P],
     "sa_head_product": [_P, _I, _L, _L, _P, _I, _P, _I, _L, _L, _I, _I, _I, _I, _I, _P, _I, _L, _P],

@@ -776,6 +776,67 @@ def paged_attention_maps(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.
     return out
 
 
+def attention_maps_heads_per_unit(num_heads: int, num_kv_heads: int) -> int:
+    """How many query heads of a key head share a unit of `paged_attention_maps_units` (a unit holds 16 rows: that
+    many heads times 16 // that many tokens)."""
+    return int(_lib.load().sa_attention_maps_heads_per_unit(int(num_heads), int(num_kv_heads)))
+
+
+def attention_maps_units_takes(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor | None, num_heads: int,
+                               maps: int = 1) -> bool:
+    """Whether `paged_attention_maps_units` takes these sizes (bfloat16 on the GPU, pages of a multiple of 16 keys, key
+    vectors of a multiple of 32 entries, values of a multiple of 16)."""
+    if q.dtype != torch.bfloat16 or not q.is_cuda or v_pages is None or k_pages.dim() != 4:
+        return False
+    _, Kh, page_size, row = k_pages.shape
+    if row % maps:
+        return False
+    return bool(_lib.load().sa_paged_attention_maps_units_takes(int(num_heads), int(Kh), int(maps), row // maps,
+                                                                int(v_pages.shape[2]), int(page_size), q.stride(0), _ptr(q)))
+
+
+def paged_attention_maps_units(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,
+                               units: torch.Tensor, unit_begin: int, unit_count: int, num_heads: int, *, scale: float,
+                               maps: int = 1, window: int | None = None,
+                               differential: "tuple[float, float, float] | None" = None, max_kv_len: int, max_q_len: int,
+                               out: torch.Tensor | None = None) -> torch.Tensor:
+    """`paged_attention_maps` in bfloat16 on the matrix cores, over the units [unit_begin, unit_begin + unit_count) of
+    `units` (int32 [U, 4]: slot, first row, tokens, first position; at most 16 // attention_maps_heads_per_unit tokens
+    each).  Two maps come with their differential combination.  Returns [T, H * dv] (rows of no unit are not written)."""
+    _dev(q, k_pages, v_pages, block_table, units, out)
+    q_stride = _rows(q, "paged_attention_maps_units: q")
+    if not attention_maps_units_takes(q, k_pages, v_pages, num_heads, maps):
+        raise KernelError("paged_attention_maps_units does not take these sizes (attention_maps_units_takes)")
+    if not k_pages.is_contiguous() or not v_pages.is_contiguous() or k_pages.dtype != q.dtype or v_pages.dtype != q.dtype:
+        raise KernelError("paged_attention_maps_units: pages are contiguous and of the queries' type")
+    num_pages, Kh, page_size, row = k_pages.shape
+    dv = v_pages.shape[2]
+    if tuple(v_pages.shape) != (num_pages, Kh, dv, page_size):
+        raise KernelError(f"paged_attention_maps_units: key pages {tuple(k_pages.shape)} do not go with value pages "
+                          f"{tuple(v_pages.shape)}")
+    if (maps == 2) != (differential is not None):
+        raise KernelError("paged_attention_maps_units: two maps come with their combination, one map has none")
+    if block_table.dim() != 2 or block_table.dtype != torch.int32 or block_table.stride(1) != 1:
+        raise KernelError("paged_attention_maps_units: block_table must be int32 [sequences, blocks]")
+    if units.dtype != torch.int32 or units.dim() != 2 or units.shape[1] != 4 or not units.is_contiguous() \
+            or unit_begin < 0 or unit_begin + unit_count > units.shape[0]:
+        raise KernelError("paged_attention_maps_units: units must be int32 [U, 4] covering the requested range")
+    if out is None:
+        out = torch.empty((q.shape[0], num_heads * dv), dtype=q.dtype, device=q.device)
+    if out.dtype != q.dtype or tuple(out.shape) != (q.shape[0], num_heads * dv):
+        raise KernelError("paged_attention_maps_units: bad output")
+    out_stride = _rows(out, "paged_attention_maps_units: out")
+    lam, eps, mult = differential if differential is not None else (0.0, 0.0, 1.0)
+    ws = _workspace(q.device)
+    for at in range(0, int(unit_count), 32768):   # (a launch takes that many units)
+        _lib.call("sa_paged_attention_maps_units", _ptr(q), q_stride, _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
+                  block_table.stride(0), _ptr(units), int(unit_begin) + at, min(32768, int(unit_count) - at), _ptr(out),
+                  out_stride, int(num_heads), Kh, row // maps, dv, page_size, int(window or 0), float(scale), int(maps),
+                  int(differential is not None), float(lam), float(eps), float(mult), int(max_kv_len), int(max_q_len),
+                  _ptr(ws), ws.numel(), _stream())
+    return out
+
+
 # --------------------------------------------------------------------------- norms behind parts, gates
 
 
@@ -929,7 +990,8 @@ def norm_rope_cache_write(proj: torch.Tensor, positions: torch.Tensor, freq: tor
                           sub: int = 1, eps: float = 0.0, q_weight: torch.Tensor | None = None, q_norm_dims: int = 0,
                           q_rot_at: int = 0, k_weight: torch.Tensor | None = None, k_norm_dims: int = 0,
                           k_rot_at: int = 0, slot_mapping: torch.Tensor | None = None,
-                          k_pages: torch.Tensor | None = None, v_pages: torch.Tensor | None = None) -> torch.Tensor:
+                          k_pages: torch.Tensor | None = None, v_pages: torch.Tensor | None = None,
+                          key_values: int = 0) -> torch.Tensor:
     """In place on fused projection rows [H * dk | K * dk | K * dv | ...]: every query and key vector is `sub` equal
     parts; in each part the first *_norm_dims entries are divided by their root mean square (eps inside the root) and
     multiplied by *_weight (None: no norm), then the entries [*_rot_at, *_rot_at + rot_dims) turn in neighbouring pairs
@@ -953,21 +1015,24 @@ def norm_rope_cache_write(proj: torch.Tensor, positions: torch.Tensor, freq: tor
             w_dtype = w.dtype
     page_size = 1
     if k_pages is not None:
-        if slot_mapping is None or (dv > 0 and v_pages is None):
+        if slot_mapping is None or ((dv > 0 or key_values > 0) and v_pages is None):
             raise KernelError("norm_rope_cache_write: key pages come with slots and, if there are values, value pages")
+        if key_values and (dv or not 0 < key_values <= dk):
+            raise KernelError("norm_rope_cache_write: key_values goes with value_dim 0 and is at most the key size")
         if k_pages.dim() != 4 or not k_pages.is_contiguous() or k_pages.dtype != proj.dtype \
                 or k_pages.shape[1] != K or k_pages.shape[3] != dk:
             raise KernelError(f"norm_rope_cache_write: key pages {tuple(k_pages.shape)} do not match {K} heads of {dk}")
         page_size = k_pages.shape[2]
-        if dv > 0 and (v_pages.dtype != proj.dtype or not v_pages.is_contiguous()
-                       or tuple(v_pages.shape) != (k_pages.shape[0], K, dv, page_size)):
+        if (dv or key_values) and (v_pages.dtype != proj.dtype or not v_pages.is_contiguous()
+                                   or tuple(v_pages.shape) != (k_pages.shape[0], K, dv or key_values, page_size)):
             raise KernelError(f"norm_rope_cache_write: value pages {tuple(v_pages.shape)} do not match")
         if slot_mapping.dtype != torch.int64 or slot_mapping.numel() < T or not slot_mapping.is_contiguous():
             raise KernelError("norm_rope_cache_write: slot_mapping must be int64 [T]")
     _lib.call("sa_norm_rope_cache_write", _ptr(proj), _code(proj), stride, _ptr(positions), _ptr(freq), int(rot_dims),
               float(rot_mult), _ptr(q_weight), int(q_norm_dims), int(q_rot_at), _ptr(k_weight), int(k_norm_dims),
               int(k_rot_at), _CODES[w_dtype] if w_dtype is not None else 0, float(eps), int(sub), _ptr(slot_mapping),
-              _ptr(k_pages), _ptr(v_pages) if dv > 0 else None, T, H, K, dk, dv, int(page_size), _stream())
+              _ptr(k_pages), _ptr(v_pages) if (dv > 0 or key_values > 0) and k_pages is not None else None, T, H, K, dk, dv,
+              int(page_size), int(key_values) if k_pages is not None else 0, _stream())
     return proj
 
 

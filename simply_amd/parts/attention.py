@@ -288,7 +288,16 @@ class DifferentialAttention(Mixer):
                                   k_weight=self.k_norm, k_norm_dims=dk if self.qk_norm else 0,
                                   slot_mapping=group.slot_mapping if write else None,
                                   k_pages=cache.k_pages if write else None, v_pages=cache.v_pages if write else None)
-        o = ops.paged_attention_maps(proj, cache.k_pages, cache.v_pages, group.block_table, ctx.token_seq,
-                                     ctx.positions, H, scale=self.scale, maps=2, window=self.window,
-                                     differential=(self.lam, self.norm_eps, 1.0 - self.diff))
+        combine = (self.lam, self.norm_eps, 1.0 - self.diff)
+        if ops.attention_maps_units_takes(proj, cache.k_pages, cache.v_pages, H, maps=2):
+            # bfloat16 at sizes that the matrix cores take: units of 16 rows (heads of a key head times tokens) per map,
+            # keys cut into ranges; the maps are combined from the ranges' 32-bit partial results
+            units, few, many, max_q = ctx.attention_units(16 // ops.attention_maps_heads_per_unit(H, K))
+            o = ops.paged_attention_maps_units(proj, cache.k_pages, cache.v_pages, group.block_table, units, 0,
+                                               few + many, H, scale=self.scale, maps=2, window=self.window,
+                                               differential=combine, max_kv_len=ctx.max_kv_len, max_q_len=max_q)
+        else:
+            o = ops.paged_attention_maps(proj, cache.k_pages, cache.v_pages, group.block_table, ctx.token_seq,
+                                         ctx.positions, H, scale=self.scale, maps=2, window=self.window,
+                                         differential=combine)
         return ops.gemm(o, self.o_proj, defer_sum=defer_sum)

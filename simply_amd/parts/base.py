@@ -97,24 +97,6 @@ class PagedKVNeed(PagedNeed):
 
 
 @dataclasses.dataclass(frozen=True)
-class PagedKeysNeed(PagedNeed):
-    """A mixer that keeps one row per token and key head and nothing else: `row_dim` entries that are scored as
-    they are, and of which a part may be read back as the token's value (a latent that stands for keys and values).
-    Pages "k" [page, kv head, page_size, row_dim], in the key layout of `PagedKVNeed`; there are no value pages."""
-
-    num_kv_heads: int
-    row_dim: int
-    window: int | None = None
-
-    def page_tensors(self, num_pages, page_size, dtype, device, fill):
-        return {"k": torch.full((num_pages, self.num_kv_heads, page_size, self.row_dim), fill, dtype=dtype,
-                                device=device)}
-
-    def bytes_per_token(self, esize):
-        return self.num_kv_heads * self.row_dim * esize
-
-
-@dataclasses.dataclass(frozen=True)
 class StateNeed:
     """A mixer that keeps a state of fixed size per request (zeroed when a request is admitted).  The manager asks
     `slot_tensor(num_slots, device)` for the storage, one row per request slot; any class with that method is

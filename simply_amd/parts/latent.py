@@ -5,7 +5,8 @@ key/value latent and r (rotated) one key part that all heads share.  Head h has 
 rotated), the key [W_uk,h c | r] and the value W_uv,h c.  Since q_h . (W_uk,h c) = (W_uk,h^T q_h) . c and
 sum_j p_j W_uv,h c_j = W_uv,h sum_j p_j c_j, the products with W_uk and W_uv move to the queries and to the result:
 attention runs with one key head whose rows are [c | r], the values are the rows' first entries, and only those
-rows are cached.
+rows are cached: once as key rows and, because the matrix cores want the keys of a value entry side by side, the
+latent once more transposed, as value pages.
 """
 from __future__ import annotations
 
@@ -14,7 +15,7 @@ import torch
 from ..config.spec import PartSpec
 from ..kernels import ops
 from ..registry import MIXERS, POSITION_ENCODINGS
-from .base import Mixer, PagedKeysNeed, ParamSpec, as_product_weight
+from .base import Mixer, PagedKVNeed, ParamSpec, as_product_weight
 
 
 @MIXERS.register("latent_attention")
@@ -69,7 +70,7 @@ class LatentAttention(Mixer):
             self.position_encoding.to_device(t["o_proj"].device)
 
     def cache_need(self):
-        return PagedKeysNeed(1, self.kv_rank + self.rot_dim, self.window)
+        return PagedKVNeed(1, self.kv_rank + self.rot_dim, self.window, self.kv_rank)
 
     def forward(self, x, ctx, cache, defer_sum=False):
         H, dk, dr, dv, Rq, R = self.num_heads, self.key_dim, self.rot_dim, self.value_dim, self.q_rank, self.kv_rank
@@ -86,9 +87,17 @@ class LatentAttention(Mixer):
             # the token's row [norm(c) | rotated r] into the pages
             ops.norm_rope_cache_write(proj[:, Rq:Rq + R + dr], ctx.positions, freq, rot_dims, 0, 1, R + dr, 0,
                                       rot_mult=mult, eps=self.norm_eps, k_weight=self.dkv_norm, k_norm_dims=R,
-                                      k_rot_at=R, slot_mapping=group.slot_mapping, k_pages=cache.k_pages)
-        o = ops.paged_attention_maps(qa, cache.k_pages, None, group.block_table, ctx.token_seq, ctx.positions, H,
-                                     scale=self.scale, value_dim=R, window=self.window)     # [T, H * R]
+                                      k_rot_at=R, slot_mapping=group.slot_mapping, k_pages=cache.k_pages,
+                                      v_pages=cache.v_pages, key_values=R)
+        if ops.attention_maps_units_takes(qa, cache.k_pages, cache.v_pages, H):
+            # bfloat16 at sizes that the matrix cores take: units of 16 rows (heads times tokens), keys cut into ranges
+            units, few, many, max_q = ctx.attention_units(16 // ops.attention_maps_heads_per_unit(H, 1))
+            o = ops.paged_attention_maps_units(qa, cache.k_pages, cache.v_pages, group.block_table, units, 0, few + many,
+                                               H, scale=self.scale, window=self.window, max_kv_len=ctx.max_kv_len,
+                                               max_q_len=max_q)
+        else:
+            o = ops.paged_attention_maps(qa, cache.k_pages, cache.v_pages, group.block_table, ctx.token_seq,
+                                         ctx.positions, H, scale=self.scale, window=self.window)     # [T, H * R]
         g_at = Rq + R + dr
         o = ops.head_product(o, self.uv, gate=proj[:, g_at:g_at + H] if self.output_gate else None)   # [T, H * dv]
         return ops.gemm(o, self.o_proj, defer_sum=defer_sum)

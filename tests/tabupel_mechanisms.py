@@ -80,8 +80,8 @@ def norm_rotation_and_pages(o, device, dtype, page_size=4, sizes=(4, 2, 10, 6, 6
 
 def latent_rows_and_pages(o, device, dtype, page_size=4, sizes=(3, 12, 8)):
     """The two uses of a latent attention: query vectors [R plain | dr rotated] without a norm, and one key row per
-    token [R normed with a weight | dr rotated, not normed] written into key-only pages; the ramp's factor is on
-    cos and sin."""
+    token [R normed with a weight | dr rotated, not normed] written into key pages and, its latent part, transposed
+    into value pages; the ramp's factor is on cos and sin."""
     import torch_ops
 
     H, R, dr = sizes
@@ -103,14 +103,18 @@ def latent_rows_and_pages(o, device, dtype, page_size=4, sizes=(3, 12, 8)):
     close(q_dev[:, :H * (R + dr)], want_q.reshape(T, -1), tol_of(dtype), "queries")
     close(q_dev[:, H * (R + dr):], qa[:, H * (R + dr):], 0.0)
     k_pages = torch.zeros((4, 1, page_size, R + dr), dtype=dtype, device=device)
+    v_pages = torch.zeros((4, 1, R, page_size), dtype=dtype, device=device)
     r_dev = row.clone().to(device)
     o.norm_rope_cache_write(r_dev[:, 5:5 + R + dr], pos.to(device), f32, dr, 0, 1, R + dr, 0, rot_mult=mult, eps=eps,
                             k_weight=w.to(device), k_norm_dims=R, k_rot_at=R, slot_mapping=slots.to(device),
-                            k_pages=k_pages)
+                            k_pages=k_pages, v_pages=v_pages, key_values=R)
     close(r_dev, row, 0.0, "the row itself stays")
     krows = torch_ops.stored_keys_as_rows(k_pages.cpu())
     for t in range(T):
-        close(krows[int(slots[t]) // page_size, 0, int(slots[t]) % page_size], want_k[t], tol_of(dtype), f"row {t}")
+        page, off = int(slots[t]) // page_size, int(slots[t]) % page_size
+        close(krows[page, 0, off], want_k[t], tol_of(dtype), f"row {t}")
+        # the latent once more, transposed, as the token's value: the very numbers of the key row
+        close(v_pages[page, 0, :, off].cpu(), krows[page, 0, off, :R], 0.0, f"value {t}")
 
 
 # --------------------------------------------------------------------------- attention over pages
@@ -400,3 +404,65 @@ def rglru_part(device, dtype, sizes=(40, 36, 3, 4), length=61, cuts=CUTS):
     for c in cuts:
         got = run_mixer(part, x.to(device), c, dtype, device)
         close(got, want, 2e-5 if dtype == torch.float32 else 6e-2, f"cuts {c[:4]}")
+
+
+# --------------------------------------------------------------------------- the same attention on the matrix cores
+
+
+def _units_of(rows, per_unit, slot, device):
+    """Consecutive positions of `rows` (sorted) grouped into units of at most per_unit tokens: (units, row of each)."""
+    units, first = [], 0
+    while first < len(rows):
+        n = 1
+        while n < per_unit and first + n < len(rows) and rows[first + n] == rows[first] + n:
+            n += 1
+        units.append([slot, first, n, rows[first]])
+        first += n
+    return torch.tensor(units, dtype=torch.int32, device=device)
+
+
+def attention_units_on_the_matrix_cores(o, device, sizes=(8, 2, 64, 128), n=700, window=100, differential=True, ranges=False):
+    """`paged_attention_maps_units` (bfloat16, pages of 16 keys) against the plain functions, with the chosen keys of
+    `differential_attention_edges`: just inside and just outside the window, at page borders and far back; the
+    queries as units of several tokens (a prompt's portion) and as units of one token (decoding), with the keys in
+    one range and cut into several."""
+    dtype, page_size = torch.bfloat16, 16
+    H, K, dk, dv = sizes
+    maps = 2 if differential else 1
+    G = H // K
+    scale, lam, eps, mult = dk ** -0.5, 0.6, 1e-5, 0.7
+    g = torch.Generator().manual_seed(15)
+    keys = torch.randn((n, K, maps, dk), generator=g, dtype=torch.float64)
+    values = torch.randn((n, K, dv), generator=g, dtype=torch.float64)
+    q = torch.randn((n, H, maps, dk), generator=g, dtype=torch.float64)
+    for win in (window, None):
+        kk = keys.clone()
+        w_ = win or n
+        rows = list(range(n - 24, n))
+        for i in rows:
+            back = [w_ - 1, w_, 1, w_ - 2][i % 4] if win else [n - 30 + i % 3, 400, i % page_size + 1, i][i % 4]
+            if i - back >= 0:
+                for h in range(H):
+                    for m in range(maps):
+                        kk[i - back, h // G, m] += q[i, h, m] * (4.0 if m == 0 else 2.0) / G
+        kd, vd, qd = kk.to(dtype).double(), values.to(dtype).double(), q.to(dtype).double()
+        want = torch.empty((n, H, dv), dtype=torch.float64)
+        for h in range(H):
+            a = [plain.windowed_softmax_attention(qd[:, h, m], kd[:, h // G, m], vd[:, h // G], scale, win) for m in range(maps)]
+            want[:, h] = plain.rms_norm(a[0] - lam * a[1], None, eps) * mult if differential else a[0]
+        k_pages, v_pages, table = _pages_of(kk.reshape(n, K, maps * dk), values, page_size, dtype, device)
+        qrows = q[rows].reshape(len(rows), H * maps * dk).to(dtype).to(device)
+        per_unit = 16 // o.attention_maps_heads_per_unit(H, K)
+        assert o.attention_maps_units_takes(qrows, k_pages, v_pages, H, maps)
+        for tokens in (per_unit, 1):
+            units = _units_of(rows, tokens, 1, device)
+            got = o.paged_attention_maps_units(qrows, k_pages, v_pages, table, units, 0, units.shape[0], H, scale=scale,
+                                               maps=maps, window=win, max_kv_len=n, max_q_len=tokens,
+                                               differential=(lam, eps, mult) if differential else None)
+            close(got, want[rows].reshape(len(rows), -1), 4e-2, f"units of {tokens}, window {win}")
+        # a single request decoding: its keys are cut into ranges over the workgroups and merged
+        units = _units_of(rows[-1:], 1, 1, device)
+        got = o.paged_attention_maps_units(qrows[-1:], k_pages, v_pages, table, units, 0, 1, H, scale=scale, maps=maps,
+                                           window=win, max_kv_len=n, max_q_len=1,
+                                           differential=(lam, eps, mult) if differential else None)
+        close(got, want[rows[-1]].reshape(1, -1), 4e-2, f"one request, window {win}")

@@ -46,6 +46,13 @@ def test_many_heads_over_one_key_head():
     mech.differential_attention_edges(ops, DEV, torch.float32, page_size=16, sizes=(18, 1, 512, 40))
 
 
+@pytest.mark.parametrize("sizes, differential", [((8, 2, 64, 128), True), ((4, 4, 32, 16), True), ((3, 1, 96, 80), True),
+                                                 ((16, 1, 160, 128), False), ((40, 1, 576, 512), False),
+                                                 ((6, 2, 64, 64), False)])
+def test_attention_units_on_the_matrix_cores(sizes, differential):
+    mech.attention_units_on_the_matrix_cores(ops, DEV, sizes=sizes, differential=differential)
+
+
 def test_recurrence_in_portions_and_other_taps():
     mech.recurrence(ops, DEV, torch.float32, cuts=(1, 2, 40, 1, 46))
     mech.recurrence(ops, DEV, torch.bfloat16, T=400, cuts=(100, 1, 129, 64, 2, 104), block=16)

@@ -40,7 +40,9 @@ def test_config_round_trip_and_spec():
     needs = [n for n, _ in model.cache_needs()]
     assert needs[0].shape == (36 * 3,) and needs[3] == needs[0]
     assert (needs[1].num_kv_heads, needs[1].head_dim, needs[1].value_dim, needs[1].window) == (2, 20, 14, 7)
-    assert (needs[2].row_dim, needs[2].window) == (24 + 8, 13) and needs[5].window is None
+    # a latent attention keeps one row [latent | rotated part] per token and the latent once more as its value
+    assert (needs[2].num_kv_heads, needs[2].head_dim, needs[2].value_dim, needs[2].window) == (1, 24 + 8, 24, 13)
+    assert needs[5].window is None
 
 
 @pytest.mark.parametrize("change, message", [

@@ -654,7 +654,7 @@ def paged_attention_maps(q, k_pages, v_pages, block_table, token_seq, positions,
 
 def norm_rope_cache_write(proj, positions, freq, rot_dims, num_heads, num_kv_heads, key_dim, value_dim, *, rot_mult=1.0,
                           sub=1, eps=0.0, q_weight=None, q_norm_dims=0, q_rot_at=0, k_weight=None, k_norm_dims=0,
-                          k_rot_at=0, slot_mapping=None, k_pages=None, v_pages=None):
+                          k_rot_at=0, slot_mapping=None, k_pages=None, v_pages=None, key_values=0):
     T = proj.shape[0]
     H, K, dk, dv = num_heads, num_kv_heads, key_dim, value_dim
     ds = dk // sub
@@ -687,10 +687,16 @@ def norm_rope_cache_write(proj, positions, freq, rot_dims, num_heads, num_kv_hea
     krows = stored_keys_as_rows(k_pages)
     krows[page, :, off] = k.reshape(T, K, dk).to(k_pages.dtype)
     k_pages.copy_(rows_as_stored_keys(krows))
+    if key_values:
+        v_pages[page, :, :, off] = k.reshape(T, K, dk)[..., :key_values].to(v_pages.dtype)
     if dv:
         v = proj[:, (H + K) * dk:(H + K) * dk + K * dv]
         v_pages[page, :, :, off] = v.reshape(T, K, dv).to(v_pages.dtype)
     return proj
+
+
+def attention_maps_units_takes(q, k_pages, v_pages, num_heads, maps=1):
+    return False
 
 
 def short_conv(x, taps, tails, seq_meta, num_seqs, max_q_len, *, in_bias=None, out_bias=None, silu=False,
