@@ -373,11 +373,13 @@ int sa_head_product(const void* x, int x_dtype, int64_t x_stride, int64_t x_head
 //   r = sigmoid(gr + r_bias), i = sigmoid(gi + i_bias), a = exp(-c r softplus(lam)),
 //   S <- a S + sqrt(1 - a^2) i u,   out = S * gelu_tanh(y + y_bias)
 // u [T, C] float32; gates [T, C / block] x [gr (block) | gi (block)] float32 (what sa_head_product leaves for the two
-// stacked gate matrices of every block); y rows of the activation type; biases and lam of vec_dtype.
+// stacked gate matrices of every block); y rows of the activation type; biases and lam of vec_dtype.  max_q_len: the
+// most tokens of a request.  Long portions run in segments of tokens side by side, through `scratch` (at least
+// num_seqs * (2 * ceil(max_q_len / 64) + 1) * C floats; null or less: one thread walks a request's channel alone).
 int sa_rglru_scan(const float* u, const float* gates, int block, const void* r_bias, const void* i_bias, const void* lam,
                   int vec_dtype, float c, const void* y, int y_dtype, int64_t y_stride, const void* y_bias,
-                  float* state, int64_t state_stride, const int* seq_meta, int num_seqs, void* out, int out_dtype,
-                  int C, hipStream_t stream);
+                  float* state, int64_t state_stride, const int* seq_meta, int num_seqs, int max_q_len, float* scratch,
+                  size_t scratch_floats, void* out, int out_dtype, int C, hipStream_t stream);
 
 // y[t, c] = silu(sum_j taps[c, j] x[t - (n - 1 - j), c]) over each request's tokens (seq_meta [S, 4]: state slot,
 // first row, rows, first position), with the inputs before the step's first row taken from tails[slot]

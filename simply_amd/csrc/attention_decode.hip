@@ -588,7 +588,8 @@ int attention_merge_ranges(const float* workspace, int num_ranges, int hd, const
                            int unit_count, int max_q_len, bf16* out, int64_t out_stride, int Kh, int G,
                            hipStream_t stream, int chunk_tiles, int group, int window, const float* sinks) {
   const int max_rows = G * max_q_len < 16 ? G * max_q_len : 16;
-  if (max_rows > 4 && num_ranges <= 64) {
+  // (the kernel of 16 threads a row walks a row's entries 64 at a time: rows of up to 256 entries)
+  if (max_rows > 4 && num_ranges <= 64 && hd <= 256) {
     paged_attention_merge_rows_kernel<<<dim3(Kh, unit_count), 256, 0, stream>>>(
         workspace, num_ranges, hd, units, unit_begin, out, out_stride, Kh, G, chunk_tiles, group, window, sinks);
     return check_launch("paged_attention_merge_rows");

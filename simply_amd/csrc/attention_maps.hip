@@ -125,7 +125,6 @@ __global__ __launch_bounds__(256) void paged_attention_maps_kernel(
           vf[t][j] = db0 + j < NDB ? *reinterpret_cast<const bf16x4*>(vp[t] + static_cast<size_t>(db0 + j) * 16 * page_size)
                                    : bf16x4{};
       floatx4 s[2] = {floatx4{0.f, 0.f, 0.f, 0.f}, floatx4{0.f, 0.f, 0.f, 0.f}};
-#pragma unroll 4
       for (int dc = 0; dc < NDC; ++dc) {
         const bf16x8 k0 = *reinterpret_cast<const bf16x8*>(kp[0] + dc * 512);
         const bf16x8 k1 = *reinterpret_cast<const bf16x8*>(kp[1] + dc * 512);

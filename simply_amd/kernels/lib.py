@@ -75,7 +75,7 @@ _SIGNATURES = {
     "sa_residual_add_next_norm": [_P, _I, _L, _F, _P, _P, _I, _F, _I, _P, _I, _I, _I, _P],
     "sa_short_conv": [_P, _I, _L, _P, _P, _I, _I, _P, _I, _I, _P, _L, _P, _I, _I, _P, _I, _I, _P],
     "sa_head_product": [_P, _I, _L, _L, _P, _I, _P, _I, _L, _L, _I, _I, _I, _I, _I, _P, _I, _L, _P],
-    "sa_rglru_scan": [_P, _P, _I, _P, _P, _P, _I, _F, _P, _I, _L, _P, _P, _L, _P, _I, _P, _I, _I, _P],
+    "sa_rglru_scan": [_P, _P, _I, _P, _P, _P, _I, _F, _P, _I, _L, _P, _P, _L, _P, _I, _I, _P, _L, _P, _I, _I, _P],
     "sa_short_conv_silu": [_P, _I, _L, _P, _I, _I, _P, _L, _P, _I, _I, _P, _I, _I, _P],
     "sa_delta_inputs_few": [_P, _I, _L, _P, _I, _I, _P, _L, _P, _I, _I, _P, _I, _I, _I, _P, _I, _L, _P, _P, _I, _I, _P, _P],
     "sa_delta_inputs_few_takes": [_I, _I],

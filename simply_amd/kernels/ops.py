@@ -1090,11 +1090,13 @@ def head_product(x: torch.Tensor, w: torch.Tensor, *, in_stride: int | None = No
 
 def rglru_scan(u: torch.Tensor, gates: torch.Tensor, block: int, r_bias: torch.Tensor, i_bias: torch.Tensor,
                lam: torch.Tensor, y: torch.Tensor, y_bias: torch.Tensor | None, state: torch.Tensor,
-               seq_meta: torch.Tensor, num_seqs: int, *, c: float = 8.0, out_dtype: torch.dtype | None = None) -> torch.Tensor:
+               seq_meta: torch.Tensor, num_seqs: int, *, c: float = 8.0, out_dtype: torch.dtype | None = None,
+               max_q_len: int | None = None) -> torch.Tensor:
     """The real-gated linear recurrence, channel by channel over each request's tokens, from and into state [slots, C]
     float32 (a view is fine): r = sigmoid(gr + r_bias), i = sigmoid(gi + i_bias), a = exp(-c r softplus(lam)),
     S <- a S + sqrt(1 - a^2) i u; returns S * gelu_tanh(y + y_bias) in out_dtype.  u float32 [T, C]; gates float32
-    [T, 2 C], per block of `block` channels [gr | gi]; y [T, C] rows of the activation type."""
+    [T, 2 C], per block of `block` channels [gr | gi]; y [T, C] rows of the activation type.  max_q_len: the most
+    tokens of a request (None: T); long portions run in segments of 64 tokens side by side."""
     _dev(u, gates, r_bias, i_bias, lam, y, y_bias, state, seq_meta)
     T, C = u.shape
     if u.dtype != torch.float32 or not u.is_contiguous() or gates.dtype != torch.float32 or not gates.is_contiguous() \
@@ -1112,9 +1114,13 @@ def rglru_scan(u: torch.Tensor, gates: torch.Tensor, block: int, r_bias: torch.T
         raise KernelError("rglru_scan: the state must be float32 [slots, >= channels]")
     _seq_meta(seq_meta, num_seqs, "rglru_scan")
     out = torch.empty((T, C), dtype=out_dtype or y.dtype, device=u.device)
+    q = max(1, min(int(max_q_len if max_q_len is not None else T), T))
+    scratch = None
+    if q > 128:   # (the segments' summaries and the requests' states at the step's start)
+        scratch = torch.empty((int(num_seqs) * (2 * -(-q // 64) + 1) * C,), dtype=torch.float32, device=u.device)
     _lib.call("sa_rglru_scan", _ptr(u), _ptr(gates), int(block), _ptr(r_bias), _ptr(i_bias), _ptr(lam), _code(lam),
               float(c), _ptr(y), _code(y), ys, _ptr(y_bias), _ptr(state), state.stride(0), _ptr(seq_meta), int(num_seqs),
-              _ptr(out), _code(out), C, _stream())
+              q, _ptr(scratch), scratch.numel() if scratch is not None else 0, _ptr(out), _code(out), C, _stream())
     return out
 
 

@@ -132,5 +132,6 @@ class RGLRU(Mixer):
                            in_bias=self.x_bias, out_bias=self.conv_bias)
         gates = ops.head_product(u, self.gate_w, out_dtype=torch.float32)
         z = ops.rglru_scan(u, gates, self.block_size, self.r_bias, self.i_bias, self.lam, proj[:, :C], self.y_bias,
-                           state, ctx.seq_meta, ctx.num_seqs, c=self.decay_mult, out_dtype=ctx.dtype)
+                           state, ctx.seq_meta, ctx.num_seqs, c=self.decay_mult, out_dtype=ctx.dtype,
+                           max_q_len=ctx.max_q_len)
         return ops.gemm(z, self.o_proj)

@@ -297,10 +297,11 @@ def recurrence(o, device, dtype, T=90, cuts=(90,), block=5):
     assert float(state[0].abs().max()) == 0.0 and float(state[1, C:].abs().max()) == 0.0
 
 
-def recurrence_of_unequal_requests(o, device, dtype):
-    """Three requests in one call (1, 40 and 7 tokens) from states that are not zero: each as alone."""
+def recurrence_of_unequal_requests(o, device, dtype, lengths=(1, 40, 7)):
+    """Three requests in one call (1, 40 and 7 tokens; or long ones, which run in segments of tokens side by side)
+    from states that are not zero: each as alone."""
     C, block = 12, 3
-    lengths, slots = (1, 40, 7), (3, 0, 2)
+    slots = (3, 0, 2)
     Tt = sum(lengths)
     u, gates = rand((Tt, C), 40).float(), rand((Tt, 2 * C), 41, 2.0).float()
     rb, ib, lam = (rand((C,), s).to(dtype) for s in (42, 43, 44))
@@ -312,7 +313,7 @@ def recurrence_of_unequal_requests(o, device, dtype):
         meta.append([s, at, L, 5])
         at += L
     got = o.rglru_scan(u.to(device), gates.to(device), block, rb.to(device), ib.to(device), lam.to(device), y.to(device),
-                       None, state, _meta(meta, device), 3, out_dtype=torch.float32)
+                       None, state, _meta(meta, device), 3, out_dtype=torch.float32, max_q_len=max(lengths))
     for s, first, L, _ in meta:
         sl = slice(first, first + L)
         g4 = gates[sl].double().view(L, C // block, 2, block)

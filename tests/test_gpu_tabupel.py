@@ -58,6 +58,10 @@ def test_recurrence_in_portions_and_other_taps():
     mech.recurrence(ops, DEV, torch.bfloat16, T=400, cuts=(100, 1, 129, 64, 2, 104), block=16)
     for n in (1, 2, 6):
         mech.short_convolution(ops, DEV, torch.float32, n=n)
+    # long portions run in segments: lengths at, just above and far from multiples of a segment, beside a single token
+    mech.recurrence_of_unequal_requests(ops, DEV, torch.float32, lengths=(1, 641, 192))
+    mech.recurrence_of_unequal_requests(ops, DEV, torch.bfloat16, lengths=(130, 129, 1000))
+    mech.recurrence(ops, DEV, torch.float32, T=1500, cuts=(700, 1, 799))
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

@@ -732,7 +732,8 @@ def head_product(x, w, *, in_stride=None, tail=0, gate=None, out_dtype=None):
     return torch.cat([o, heads[..., I:]], dim=-1).reshape(T, H * (O + tail)).to(out_dtype or x.dtype)
 
 
-def rglru_scan(u, gates, block, r_bias, i_bias, lam, y, y_bias, state, seq_meta, num_seqs, *, c=8.0, out_dtype=None):
+def rglru_scan(u, gates, block, r_bias, i_bias, lam, y, y_bias, state, seq_meta, num_seqs, *, c=8.0, out_dtype=None,
+               max_q_len=None):
     T, C = u.shape
     g = _f(gates).reshape(T, C // block, 2, block)
     r = torch.sigmoid(g[:, :, 0].reshape(T, C) + _f(r_bias))
