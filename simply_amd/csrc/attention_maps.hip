@@ -22,6 +22,7 @@ namespace sa {
 
 int paged_attention_decode_ranges(int seq_count, int Kh, int window, int max_kv_len, int num_splits);
 
+constexpr int kKeyBatch = 6;           // key blocks of 32 entries whose loads are asked for together
 constexpr int kMapsSubTiles = 2048;   // sub-tiles of 16 keys whose page a workgroup looks up at a time
 
 struct MapsShape {
@@ -125,12 +126,25 @@ __global__ __launch_bounds__(256) void paged_attention_maps_kernel(
           vf[t][j] = db0 + j < NDB ? *reinterpret_cast<const bf16x4*>(vp[t] + static_cast<size_t>(db0 + j) * 16 * page_size)
                                    : bf16x4{};
       floatx4 s[2] = {floatx4{0.f, 0.f, 0.f, 0.f}, floatx4{0.f, 0.f, 0.f, 0.f}};
-      for (int dc = 0; dc < NDC; ++dc) {
-        const bf16x8 k0 = *reinterpret_cast<const bf16x8*>(kp[0] + dc * 512);
-        const bf16x8 k1 = *reinterpret_cast<const bf16x8*>(kp[1] + dc * 512);
-        const bf16x8 qf = q_s[dc * kWave + lane];
-        s[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k0, qf, s[0], 0, 0, 0);
-        s[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k1, qf, s[1], 0, 0, 0);
+      // the key blocks in batches of kKeyBatch: a batch's loads are all asked for before its first product, so a wave
+      // waits for memory once a batch and not once a block (a block beyond the vector's last is the last one again,
+      // loaded and not used: every load of a batch is unconditional)
+      for (int dc0 = 0; dc0 < NDC; dc0 += kKeyBatch) {
+        bf16x8 kf[2][kKeyBatch];
+#pragma unroll
+        for (int j = 0; j < kKeyBatch; ++j) {
+          const int dc = dc0 + j < NDC ? dc0 + j : NDC - 1;
+          kf[0][j] = *reinterpret_cast<const bf16x8*>(kp[0] + dc * 512);
+          kf[1][j] = *reinterpret_cast<const bf16x8*>(kp[1] + dc * 512);
+        }
+#pragma unroll
+        for (int j = 0; j < kKeyBatch; ++j) {
+          if (dc0 + j < NDC) {
+            const bf16x8 qf = q_s[(dc0 + j) * kWave + lane];
+            s[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[0][j], qf, s[0], 0, 0, 0);
+            s[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[1][j], qf, s[1], 0, 0, 0);
+          }
+        }
       }
       // ---- scale, mask, online softmax.  Lane (row r, grp) holds keys sk0 + 4 * grp + v of each sub-tile.
       float p[2][4];

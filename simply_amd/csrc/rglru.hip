@@ -76,6 +76,49 @@ __global__ __launch_bounds__(256) void head_product_kernel(
   }
 }
 
+// The same product for a handful of tokens (decoding): a wave per (head, output) holds up to kHpFewTokens tokens'
+// sums in its lanes, every lane over the inputs lane, lane + 64, ..., and adds the lanes up at the end, so the
+// weights are streamed once in contiguous pieces by as many waves as there are outputs.
+constexpr int kHpFewTokens = 8;
+__global__ __launch_bounds__(256) void head_product_few_kernel(
+    const void* __restrict__ x, int x_dtype, int64_t x_stride, int64_t x_head_stride, const void* __restrict__ w,
+    int w_dtype, void* __restrict__ out, int out_dtype, int64_t out_stride, int64_t out_head_stride, int T, int I, int O,
+    int tail, const void* __restrict__ gate, int gate_dtype, int64_t gate_stride) {
+  const int lane = threadIdx.x % kWave, o = blockIdx.x * 4 + threadIdx.x / kWave, h = blockIdx.y;
+  const int t0 = blockIdx.z * kHpFewTokens;
+  if (o >= O) return;   // (a whole wave)
+  const size_t wb = (static_cast<size_t>(h) * O + o) * I;
+  float acc[kHpFewTokens];
+#pragma unroll
+  for (int k = 0; k < kHpFewTokens; ++k) acc[k] = 0.f;
+  for (int i = lane; i < I; i += kWave) {
+    const float wv = load_f(w, w_dtype, wb + i);
+#pragma unroll
+    for (int k = 0; k < kHpFewTokens; ++k) {
+      const int t = t0 + k < T ? t0 + k : T - 1;
+      acc[k] = fmaf(load_f(x, x_dtype, static_cast<size_t>(t) * x_stride + static_cast<size_t>(h) * x_head_stride + i), wv,
+                    acc[k]);
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < kHpFewTokens; ++k) {
+    const float v = wave_sum(acc[k]);
+    const int t = t0 + k;
+    if (t >= T) continue;
+    const size_t ob = static_cast<size_t>(t) * out_stride + static_cast<size_t>(h) * out_head_stride;
+    if (lane == 0) {
+      const float gv = gate != nullptr
+                           ? 1.f / (1.f + expf(-load_f(gate, gate_dtype, static_cast<size_t>(t) * gate_stride + h)))
+                           : 1.f;
+      store_f(out, out_dtype, ob + o, v * gv);
+    }
+    if (o == 0) {
+      const size_t xb = static_cast<size_t>(t) * x_stride + static_cast<size_t>(h) * x_head_stride + I;
+      for (int e = lane; e < tail; e += kWave) store_f(out, out_dtype, ob + O + e, load_f(x, x_dtype, xb + e));
+    }
+  }
+}
+
 // The recurrence of one channel over the tokens [j0, j1) of a request from the state S: the loads of eight tokens are
 // asked for together, the recurrence itself is one multiply-add a token.  kOut: results are written; else only the
 // state and the product of the decays come back (a segment's summary).
@@ -211,6 +254,12 @@ extern "C" int sa_head_product(const void* x, int x_dtype, int64_t x_stride, int
   SA_REQUIRE(gate == nullptr || gate_stride >= H, "head_product: the gates' row stride is below the heads");
   const int tiles = (T + kHpTokens - 1) / kHpTokens, cols = (O + kHpOutputs - 1) / kHpOutputs;
   SA_REQUIRE(H <= 65535 && cols <= 65535, "head_product: too many heads or outputs");
+  if (T <= 2 * kHpFewTokens && (O + 3) / 4 <= 65535) {
+    head_product_few_kernel<<<dim3((O + 3) / 4, H, (T + kHpFewTokens - 1) / kHpFewTokens), 256, 0, stream>>>(
+        x, x_dtype, x_stride, x_head_stride, w, w_dtype, out, out_dtype, out_stride, out_head_stride, T, I, O, tail, gate,
+        gate_dtype, gate_stride);
+    return check_launch("head_product_few");
+  }
   head_product_kernel<<<dim3(tiles, H, cols), 256, 0, stream>>>(x, x_dtype, x_stride, x_head_stride, w, w_dtype, out,
                                                                 out_dtype, out_stride, out_head_stride, T, I, O, tail,
                                                                 gate, gate_dtype, gate_stride);
