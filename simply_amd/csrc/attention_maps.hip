@@ -22,7 +22,6 @@ namespace sa {
 
 int paged_attention_decode_ranges(int seq_count, int Kh, int window, int max_kv_len, int num_splits);
 
-constexpr int kKeyBatch = 6;           // key blocks of 32 entries whose loads are asked for together
 constexpr int kMapsSubTiles = 2048;   // sub-tiles of 16 keys whose page a workgroup looks up at a time
 
 struct MapsShape {
@@ -32,8 +31,10 @@ struct MapsShape {
   float scale;
 };
 
-// NDBW: blocks of 16 value entries that a wave owns (its quarter of them, rounded up)
-template <int NDBW>
+// NDBW: blocks of 16 value entries that a wave owns (its quarter of them, rounded up).  KB: key blocks of 32 entries
+// whose loads are asked for together (0: block by block, for launches with many workgroups on a CU, whose waits cover
+// one another; with a few workgroups on the GPU a wave waits for memory once a batch instead of once a block).
+template <int NDBW, int KB>
 __global__ __launch_bounds__(256) void paged_attention_maps_kernel(
     const bf16* __restrict__ q, int64_t q_stride, const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
     const int* __restrict__ block_table, int table_stride, const SeqMeta* __restrict__ units, int unit_begin,
@@ -126,23 +127,32 @@ __global__ __launch_bounds__(256) void paged_attention_maps_kernel(
           vf[t][j] = db0 + j < NDB ? *reinterpret_cast<const bf16x4*>(vp[t] + static_cast<size_t>(db0 + j) * 16 * page_size)
                                    : bf16x4{};
       floatx4 s[2] = {floatx4{0.f, 0.f, 0.f, 0.f}, floatx4{0.f, 0.f, 0.f, 0.f}};
-      // the key blocks in batches of kKeyBatch: a batch's loads are all asked for before its first product, so a wave
-      // waits for memory once a batch and not once a block (a block beyond the vector's last is the last one again,
-      // loaded and not used: every load of a batch is unconditional)
-      for (int dc0 = 0; dc0 < NDC; dc0 += kKeyBatch) {
-        bf16x8 kf[2][kKeyBatch];
-#pragma unroll
-        for (int j = 0; j < kKeyBatch; ++j) {
-          const int dc = dc0 + j < NDC ? dc0 + j : NDC - 1;
-          kf[0][j] = *reinterpret_cast<const bf16x8*>(kp[0] + dc * 512);
-          kf[1][j] = *reinterpret_cast<const bf16x8*>(kp[1] + dc * 512);
+      if constexpr (KB == 0) {
+        for (int dc = 0; dc < NDC; ++dc) {
+          const bf16x8 k0 = *reinterpret_cast<const bf16x8*>(kp[0] + dc * 512);
+          const bf16x8 k1 = *reinterpret_cast<const bf16x8*>(kp[1] + dc * 512);
+          const bf16x8 qf = q_s[dc * kWave + lane];
+          s[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k0, qf, s[0], 0, 0, 0);
+          s[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k1, qf, s[1], 0, 0, 0);
         }
+      } else {
+        // (a block beyond the vector's last is the last one again, loaded and not used: every load of a batch is
+        // unconditional)
+        for (int dc0 = 0; dc0 < NDC; dc0 += KB) {
+          bf16x8 kf[2][KB > 0 ? KB : 1];
 #pragma unroll
-        for (int j = 0; j < kKeyBatch; ++j) {
-          if (dc0 + j < NDC) {
-            const bf16x8 qf = q_s[(dc0 + j) * kWave + lane];
-            s[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[0][j], qf, s[0], 0, 0, 0);
-            s[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[1][j], qf, s[1], 0, 0, 0);
+          for (int j = 0; j < KB; ++j) {
+            const int dc = dc0 + j < NDC ? dc0 + j : NDC - 1;
+            kf[0][j] = *reinterpret_cast<const bf16x8*>(kp[0] + dc * 512);
+            kf[1][j] = *reinterpret_cast<const bf16x8*>(kp[1] + dc * 512);
+          }
+#pragma unroll
+          for (int j = 0; j < KB; ++j) {
+            if (dc0 + j < NDC) {
+              const bf16x8 qf = q_s[(dc0 + j) * kWave + lane];
+              s[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[0][j], qf, s[0], 0, 0, 0);
+              s[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[1][j], qf, s[1], 0, 0, 0);
+            }
           }
         }
       }
@@ -352,14 +362,21 @@ extern "C" int sa_paged_attention_maps_units(const void* q, int64_t q_stride, co
   const SeqMeta* um = reinterpret_cast<const SeqMeta*>(units);
   bf16* op = static_cast<bf16*>(out);
   float* ws = static_cast<float*>(workspace);
-#define SA_LAUNCH(N)                                                                                                  \
-  paged_attention_maps_kernel<N><<<grid, 256, smem, stream>>>(qp, q_stride, kp, vp, block_table, table_stride, um,    \
-                                                              unit_begin, op, out_stride, sh, ws, partial ? 1 : 0)
-  if (per_wave <= 1) SA_LAUNCH(1);
-  else if (per_wave <= 2) SA_LAUNCH(2);
-  else if (per_wave <= 4) SA_LAUNCH(4);
-  else if (per_wave <= 8) SA_LAUNCH(8);
-  else SA_LAUNCH(16);
+#define SA_LAUNCH_KB(N, B)                                                                                            \
+  paged_attention_maps_kernel<N, B><<<grid, 256, smem, stream>>>(qp, q_stride, kp, vp, block_table, table_stride, um, \
+                                                                 unit_begin, op, out_stride, sh, ws, partial ? 1 : 0)
+  // few workgroups for the GPU's 256 CUs: the key blocks' loads in batches
+  const int batch = static_cast<int64_t>(KS) * KhV * unit_count > 1024 ? 0 : sh.ndc <= 2 ? 2 : 6;
+#define SA_LAUNCH(N)                   \
+  if (batch == 0) SA_LAUNCH_KB(N, 0);  \
+  else if (batch == 2) SA_LAUNCH_KB(N, 2); \
+  else SA_LAUNCH_KB(N, 6)
+  if (per_wave <= 1) { SA_LAUNCH(1); }
+  else if (per_wave <= 2) { SA_LAUNCH(2); }
+  else if (per_wave <= 4) { SA_LAUNCH(4); }
+  else if (per_wave <= 8) { SA_LAUNCH(8); }
+  else { SA_LAUNCH(16); }
+#undef SA_LAUNCH_KB
 #undef SA_LAUNCH
   if (check_launch("paged_attention_maps_units")) return 1;
   const int max_rows = Gc * max_q_len < 16 ? Gc * max_q_len : 16;
