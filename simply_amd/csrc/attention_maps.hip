@@ -366,11 +366,12 @@ extern "C" int sa_paged_attention_maps_units(const void* q, int64_t q_stride, co
   paged_attention_maps_kernel<N, B><<<grid, 256, smem, stream>>>(qp, q_stride, kp, vp, block_table, table_stride, um, \
                                                                  unit_begin, op, out_stride, sh, ws, partial ? 1 : 0)
   // few workgroups for the GPU's 256 CUs: the key blocks' loads in batches
-  const int batch = static_cast<int64_t>(KS) * KhV * unit_count > 1024 ? 0 : sh.ndc <= 2 ? 2 : 6;
+  const int batch = static_cast<int64_t>(KS) * KhV * unit_count > 1024 ? 0 : sh.ndc <= 2 ? 2 : sh.ndc <= 12 ? 6 : 18;
 #define SA_LAUNCH(N)                   \
   if (batch == 0) SA_LAUNCH_KB(N, 0);  \
   else if (batch == 2) SA_LAUNCH_KB(N, 2); \
-  else SA_LAUNCH_KB(N, 6)
+  else if (batch == 6) SA_LAUNCH_KB(N, 6); \
+  else SA_LAUNCH_KB(N, 18)
   if (per_wave <= 1) { SA_LAUNCH(1); }
   else if (per_wave <= 2) { SA_LAUNCH(2); }
   else if (per_wave <= 4) { SA_LAUNCH(4); }
