@@ -313,10 +313,12 @@ __global__ __launch_bounds__(kWave) void norm_rope_cache_write_kernel(
       for (int j = 0; j < kPartPerLane; ++j) {
         const int i = lane + j * kWave;
         raw[j] = other[j] = 0.f;
-        if (i < ds) {
-          raw[j] = to_float(src[i]);
+        if (j * kWave < ds && i < ds) {   // (the first test is uniform: pieces beyond the part cost a branch)
           const int e = i - hn.rot_at;
-          if (e >= 0 && e < rot_dims) other[j] = to_float(src[hn.rot_at + (e ^ 1)]);
+          const bool turns = e >= 0 && e < rot_dims;
+          // a query entry that is neither normed nor rotated stays where it is: it is not even read
+          if (!is_q || turns || (hn.w != nullptr && i < hn.norm_dims)) raw[j] = to_float(src[i]);
+          if (turns) other[j] = to_float(src[hn.rot_at + (e ^ 1)]);
           if (i < hn.norm_dims) ss = fmaf(raw[j], raw[j], ss);
         }
       }
@@ -329,7 +331,8 @@ __global__ __launch_bounds__(kWave) void norm_rope_cache_write_kernel(
 #pragma unroll
       for (int j = 0; j < kPartPerLane; ++j) {
         const int i = lane + j * kWave;
-        if (i >= ds) continue;
+        if (j * kWave >= ds || i >= ds) continue;
+        if (is_q && (i - hn.rot_at < 0 || i - hn.rot_at >= rot_dims) && !(hn.w != nullptr && i < hn.norm_dims)) continue;
         float v = raw[j];
         if (hn.w != nullptr && i < hn.norm_dims) v = v * r * load_f(hn.w, w_dtype, i);
         const int e = i - hn.rot_at;
