@@ -278,7 +278,8 @@ struct HeadNormRope {
   int norm_dims, rot_at;
 };
 constexpr int kPartPerLane = 16;  // parts of up to 1024 entries
-template <typename T>
+// NP: pieces of 64 entries that a lane holds of a part (registers for no more than the part needs)
+template <typename T, int NP>
 __global__ __launch_bounds__(kWave) void norm_rope_cache_write_kernel(
     T* __restrict__ proj, int64_t row_stride, const int* __restrict__ positions, const float* __restrict__ freq,
     int rot_dims, float rot_mult, HeadNormRope qn, HeadNormRope kn, int w_dtype, float eps, int sub,
@@ -307,10 +308,10 @@ __global__ __launch_bounds__(kWave) void norm_rope_cache_write_kernel(
     }
     for (int part = 0; part < sub; ++part) {
       T* src = row + static_cast<size_t>(head) * dk + static_cast<size_t>(part) * ds;
-      float raw[kPartPerLane], other[kPartPerLane];
+      float raw[NP], other[NP];
       float ss = 0.f;
 #pragma unroll
-      for (int j = 0; j < kPartPerLane; ++j) {
+      for (int j = 0; j < NP; ++j) {
         const int i = lane + j * kWave;
         raw[j] = other[j] = 0.f;
         if (j * kWave < ds && i < ds) {   // (the first test is uniform: pieces beyond the part cost a branch)
@@ -329,7 +330,7 @@ __global__ __launch_bounds__(kWave) void norm_rope_cache_write_kernel(
       }
       // (every lane has read what it needs of the part before any lane writes: the wave runs in lockstep)
 #pragma unroll
-      for (int j = 0; j < kPartPerLane; ++j) {
+      for (int j = 0; j < NP; ++j) {
         const int i = lane + j * kWave;
         if (j * kWave >= ds || i >= ds) continue;
         if (is_q && (i - hn.rot_at < 0 || i - hn.rot_at >= rot_dims) && !(hn.w != nullptr && i < hn.norm_dims)) continue;
@@ -515,15 +516,26 @@ extern "C" int sa_norm_rope_cache_write(void* proj, int dtype, int64_t row_strid
   SA_REQUIRE(H + 2 * K <= 65535, "norm_rope_cache_write: too many heads");
   const dim3 grid(T, H + K + (dv > 0 ? K : 0));
   const HeadNormRope qn{q_weight, q_norm_dims, q_rot_at}, kn{k_weight, k_norm_dims, k_rot_at};
-  if (dtype == kF32)
-    norm_rope_cache_write_kernel<float><<<grid, kWave, 0, stream>>>(
-        static_cast<float*>(proj), row_stride, positions, freq, rot_dims, rot_mult, qn, kn, w_dtype, eps, sub,
-        slot_mapping, static_cast<float*>(k_pages), static_cast<float*>(v_pages), H, K, dk, dv, page_size, key_values);
-  else if (dtype == kBF16)
-    norm_rope_cache_write_kernel<bf16><<<grid, kWave, 0, stream>>>(
-        static_cast<bf16*>(proj), row_stride, positions, freq, rot_dims, rot_mult, qn, kn, w_dtype, eps, sub,
-        slot_mapping, static_cast<bf16*>(k_pages), static_cast<bf16*>(v_pages), H, K, dk, dv, page_size, key_values);
-  else
-    SA_REQUIRE(false, "norm_rope_cache_write: unknown dtype %d", dtype);
+  SA_REQUIRE(dtype == kF32 || dtype == kBF16, "norm_rope_cache_write: unknown dtype %d", dtype);
+#define SA_LAUNCH(NP)                                                                                                 \
+  do {                                                                                                                \
+    if (dtype == kF32)                                                                                                \
+      norm_rope_cache_write_kernel<float, NP><<<grid, kWave, 0, stream>>>(                                            \
+          static_cast<float*>(proj), row_stride, positions, freq, rot_dims, rot_mult, qn, kn, w_dtype, eps, sub,      \
+          slot_mapping, static_cast<float*>(k_pages), static_cast<float*>(v_pages), H, K, dk, dv, page_size,          \
+          key_values);                                                                                                \
+    else                                                                                                              \
+      norm_rope_cache_write_kernel<bf16, NP><<<grid, kWave, 0, stream>>>(                                             \
+          static_cast<bf16*>(proj), row_stride, positions, freq, rot_dims, rot_mult, qn, kn, w_dtype, eps, sub,       \
+          slot_mapping, static_cast<bf16*>(k_pages), static_cast<bf16*>(v_pages), H, K, dk, dv, page_size,            \
+          key_values);                                                                                                \
+  } while (0)
+  const int pieces = (ds + kWave - 1) / kWave;
+  if (pieces <= 1) SA_LAUNCH(1);
+  else if (pieces <= 2) SA_LAUNCH(2);
+  else if (pieces <= 4) SA_LAUNCH(4);
+  else if (pieces <= 9) SA_LAUNCH(9);
+  else SA_LAUNCH(16);
+#undef SA_LAUNCH
   return check_launch("norm_rope_cache_write");
 }
