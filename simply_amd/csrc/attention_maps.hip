@@ -23,6 +23,7 @@ namespace sa {
 int paged_attention_decode_ranges(int seq_count, int Kh, int window, int max_kv_len, int num_splits);
 
 constexpr int kMapsSubTiles = 2048;   // sub-tiles of 16 keys whose page a workgroup looks up at a time
+constexpr int kWaveUnitsFrom = 2048;  // (units x heads) from which a wave takes a unit of its own
 
 struct MapsShape {
   int Kh, maps, chunks, Gc, G_all;   // key heads; maps per head; chunks of Gc query heads per key head (G_all in all)
@@ -239,6 +240,159 @@ __global__ __launch_bounds__(256) void paged_attention_maps_kernel(
   }
 }
 
+// The same attention for launches with many units (portions of prompts): every wave of a workgroup takes a unit of
+// its own, four consecutive units a workgroup (fewer where the waves' queries would not fit into LDS), and owns all of its value entries, so the scores are computed once.  The
+// four waves walk nearly the same keys at nearly the same time (consecutive tokens of a request), so the key blocks that
+// one of them brings come from the CU's cache for the others.  No ranges of keys, no barrier: a wave looks its pages up
+// itself, sub-tile by sub-tile, and waves of other workgroups cover that wait.
+// NDBT: blocks of 16 value entries (rounded up to a power of two; those beyond the values' are skipped).
+constexpr int kValueBatch = 8;   // value blocks whose loads are asked for together
+template <int NDBT>
+__global__ __launch_bounds__(256) void paged_attention_maps_waves_kernel(
+    const bf16* __restrict__ q, int64_t q_stride, const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
+    const int* __restrict__ block_table, int table_stride, const SeqMeta* __restrict__ units, int unit_begin,
+    int unit_count, bf16* __restrict__ out, int64_t out_stride, MapsShape sh, float* __restrict__ workspace,
+    int always_partial) {
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  const int tid = threadIdx.x, lane = tid % kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const int u = blockIdx.z * (blockDim.x / kWave) + wave, vy = blockIdx.y, KhV = gridDim.y;   // (four waves, or as many as LDS holds)
+  if (u >= unit_count) return;   // (a whole wave; nothing below waits for another wave)
+  const int r = lane % 16, grp = lane / 16;
+  const int chunk = vy % sh.chunks, map = (vy / sh.chunks) % sh.maps, kh = vy / (sh.chunks * sh.maps);
+  const SeqMeta sm = units[unit_begin + u];
+  const int Gc = sh.Gc, NDC = sh.ndc, HDV = sh.hdv, page_size = sh.page_size, window = sh.window;
+  const int NDB = HDV / 16;
+  const int rows = Gc * sm.q_len;
+  if (rows == 0) return;
+  bf16x8* q_s = reinterpret_cast<bf16x8*>(smem_raw) + static_cast<size_t>(wave) * NDC * kWave;   // this wave's own
+  const int* table = block_table + static_cast<size_t>(sm.slot) * table_stride;
+  const int qi = r / Gc, g = r % Gc;
+  const bool row_ok = r < rows;
+  const int pos_r = sm.pos0 + qi;
+  const int hi = sm.pos0 + sm.q_len;
+  const int lo = (window > 0 && sm.pos0 - window + 1 > 0) ? sm.pos0 - window + 1 : 0;
+  const int lo_r = (window > 0 && pos_r - window + 1 > 0) ? pos_r - window + 1 : 0;
+  {
+    const int head = kh * sh.G_all + chunk * Gc + (row_ok ? g : 0);
+    const bf16* qp = q + static_cast<size_t>(sm.q_start + (row_ok ? qi : 0)) * q_stride +
+                     (static_cast<size_t>(head) * sh.maps + map) * (NDC * 32) + grp * 8;
+    for (int dc = 0; dc < NDC; ++dc)
+      q_s[dc * kWave + lane] = row_ok ? *reinterpret_cast<const bf16x8*>(qp + dc * 32) : bf16x8{};
+  }
+  const int safe_page = table[(hi - 1) / page_size];   // the unit's last token has a page: loads that are not needed go there
+  floatx4 acc[NDBT];
+#pragma unroll
+  for (int j = 0; j < NDBT; ++j) acc[j] = floatx4{0.f, 0.f, 0.f, 0.f};
+  float m_run = -INFINITY, l_run = 0.f;
+  const size_t row_elems = static_cast<size_t>(sh.row_blocks) * 32;
+
+  for (int tile = lo / kTile; tile * kTile < hi; ++tile) {
+    const int key0 = tile * kTile;
+    bool sub_ok[2];
+    const bf16* kp[2];
+    const bf16* vp[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const int sk0 = key0 + t * 16;
+      sub_ok[t] = sk0 < hi && sk0 + 16 > lo;   // wave-uniform
+      const int block = sk0 / page_size;
+      const int page = sub_ok[t] ? table[block] : safe_page;
+      const int blk = sub_ok[t] ? (sk0 - block * page_size) / 16 : 0;
+      const size_t head = static_cast<size_t>(page) * sh.Kh + kh;
+      kp[t] = k_pages + head * page_size * row_elems + static_cast<size_t>(blk) * (sh.row_blocks * 512) +
+              static_cast<size_t>(map * NDC) * 512 + lane * 8;
+      vp[t] = v_pages + (head * HDV + r) * page_size + blk * 16 + grp * 4;
+    }
+    floatx4 s[2] = {floatx4{0.f, 0.f, 0.f, 0.f}, floatx4{0.f, 0.f, 0.f, 0.f}};
+    for (int dc = 0; dc < NDC; ++dc) {
+      const bf16x8 k0 = *reinterpret_cast<const bf16x8*>(kp[0] + dc * 512);
+      const bf16x8 k1 = *reinterpret_cast<const bf16x8*>(kp[1] + dc * 512);
+      const bf16x8 qf = q_s[dc * kWave + lane];
+      s[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k0, qf, s[0], 0, 0, 0);
+      s[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k1, qf, s[1], 0, 0, 0);
+    }
+    float p[2][4];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const int key = key0 + t * 16 + grp * 4 + v;
+        const bool vis = sub_ok[t] && row_ok && key <= pos_r && key >= lo_r;
+        const float x = vis ? s[t][v] * sh.scale : -INFINITY;
+        p[t][v] = x;
+        mx = fmaxf(mx, x);
+      }
+    mx = max_over_row_lanes(mx);
+    const float m_new = fmaxf(m_run, mx);
+    const float alpha = m_new == -INFINITY ? 1.f : __expf(m_run - m_new);
+    float psum = 0.f;
+    bf16x8 pf;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const float e = p[t][v] == -INFINITY ? 0.f : __expf(p[t][v] - m_new);
+        psum += e;
+        pf[t * 4 + v] = to_bf16_raw(e);
+      }
+    l_run = l_run * alpha + psum;
+    m_run = m_new;
+    const bool tail = key0 + kTile > hi || !sub_ok[0] || !sub_ok[1];
+#pragma unroll
+    for (int j0 = 0; j0 < NDBT; j0 += kValueBatch) {
+      constexpr int kB = NDBT < kValueBatch ? NDBT : kValueBatch;
+      bf16x4 vf[2][kB];
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int j = 0; j < kB; ++j)
+          vf[t][j] = j0 + j < NDB ? *reinterpret_cast<const bf16x4*>(vp[t] + static_cast<size_t>(j0 + j) * 16 * page_size)
+                                  : bf16x4{};
+#pragma unroll
+      for (int j = 0; j < kB; ++j) {
+        bf16x8 a;
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int v = 0; v < 4; ++v) a[t * 4 + v] = vf[t][j][v];
+        if (tail) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const int key = key0 + (e / 4) * 16 + grp * 4 + (e % 4);
+            if (key >= hi || !sub_ok[e / 4]) a[e] = to_bf16_raw(0.f);
+          }
+        }
+#pragma unroll
+        for (int v = 0; v < 4; ++v) acc[j0 + j][v] *= alpha;
+        acc[j0 + j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, pf, acc[j0 + j], 0, 0, 0);
+      }
+    }
+  }
+  l_run = sum_over_row_lanes(l_run);
+  if (!row_ok) return;
+  if (!always_partial) {
+    bf16* op = out + static_cast<size_t>(sm.q_start + qi) * out_stride + static_cast<size_t>(vy * Gc + g) * HDV;
+    const float inv = 1.f / l_run;
+#pragma unroll
+    for (int j = 0; j < NDBT; ++j)
+      if (j < NDB)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) op[j * 16 + 4 * grp + v] = float_to_bf16(acc[j][v] * inv);
+    return;
+  }
+  const size_t row_words = HDV + kRowExtra;
+  float* wp = workspace + ((static_cast<size_t>(u) * KhV + vy) * 16 + r) * row_words;   // (one range of keys)
+#pragma unroll
+  for (int j = 0; j < NDBT; ++j)
+    if (j < NDB) *reinterpret_cast<floatx4*>(wp + j * 16 + 4 * grp) = acc[j];
+  if (grp == 0) {
+    wp[HDV] = m_run;
+    wp[HDV + 1] = l_run;
+  }
+}
+
 // The differential combination from the partial results of two maps: per (unit, key head, chunk, row) both maps'
 // ranges are added up in their order, o = a_1 - lambda a_2 is divided by its root mean square over the head's values
 // and multiplied by mult.  One workgroup per row and (key head, chunk); a thread takes the value entries tid,
@@ -353,15 +507,37 @@ extern "C" int sa_paged_attention_maps_units(const void* q, int64_t q_stride, co
   const bool partial = differential != 0;
   SA_REQUIRE(!(partial || KS > 1) || (workspace != nullptr && per_split * KS <= workspace_bytes),
              "paged_attention_maps_units: the partial results (%zu bytes) do not fit the workspace", per_split * KS);
-  const dim3 grid(KS, KhV, unit_count);
-  const size_t smem = static_cast<size_t>(sh.ndc) * kWave * sizeof(bf16x8);
-  const int per_wave = (hd_v / 16 + 3) / 4;
   const bf16* qp = static_cast<const bf16*>(q);
   const bf16* kp = static_cast<const bf16*>(k_pages);
   const bf16* vp = static_cast<const bf16*>(v_pages);
   const SeqMeta* um = reinterpret_cast<const SeqMeta*>(units);
   bf16* op = static_cast<bf16*>(out);
   float* ws = static_cast<float*>(workspace);
+  // many units (portions of prompts) and one range of keys: a wave per unit, if four waves' queries fit into LDS
+  int waves = 4;
+  while (waves > 1 && static_cast<size_t>(waves) * sh.ndc * kWave * sizeof(bf16x8) > 64 * 1024) --waves;
+  const size_t smem_waves = static_cast<size_t>(waves) * sh.ndc * kWave * sizeof(bf16x8);
+  // (values of up to 128 entries: with wider ones a wave's accumulators leave room for two waves on a SIMD, and 2,048
+  // units of a latent attention's 512 entries took 832 us so against 595 us with four waves a unit)
+  if (KS == 1 && static_cast<int64_t>(unit_count) * KhV >= kWaveUnitsFrom && smem_waves <= 64 * 1024 && hd_v <= 128) {
+    const dim3 grid(1, KhV, (unit_count + waves - 1) / waves);
+    const int ndb = hd_v / 16;
+#define SA_LAUNCH_W(N)                                                                                             \
+  paged_attention_maps_waves_kernel<N><<<grid, waves * kWave, smem_waves, stream>>>(qp, q_stride, kp, vp, block_table, \
+                                                                         table_stride, um, unit_begin, unit_count, \
+                                                                         op, out_stride, sh, ws, partial ? 1 : 0)
+    if (ndb <= 1) SA_LAUNCH_W(1);
+    else if (ndb <= 2) SA_LAUNCH_W(2);
+    else if (ndb <= 4) SA_LAUNCH_W(4);
+    else if (ndb <= 8) SA_LAUNCH_W(8);
+    else if (ndb <= 16) SA_LAUNCH_W(16);
+    else if (ndb <= 32) SA_LAUNCH_W(32);
+    else SA_LAUNCH_W(64);
+#undef SA_LAUNCH_W
+  } else {
+  const dim3 grid(KS, KhV, unit_count);
+  const size_t smem = static_cast<size_t>(sh.ndc) * kWave * sizeof(bf16x8);
+  const int per_wave = (hd_v / 16 + 3) / 4;
 #define SA_LAUNCH_KB(N, B)                                                                                            \
   paged_attention_maps_kernel<N, B><<<grid, 256, smem, stream>>>(qp, q_stride, kp, vp, block_table, table_stride, um, \
                                                                  unit_begin, op, out_stride, sh, ws, partial ? 1 : 0)
@@ -379,6 +555,7 @@ extern "C" int sa_paged_attention_maps_units(const void* q, int64_t q_stride, co
   else { SA_LAUNCH(16); }
 #undef SA_LAUNCH_KB
 #undef SA_LAUNCH
+  }
   if (check_launch("paged_attention_maps_units")) return 1;
   const int max_rows = Gc * max_q_len < 16 ? Gc * max_q_len : 16;
   if (partial) {

@@ -422,11 +422,12 @@ def _units_of(rows, per_unit, slot, device):
     return torch.tensor(units, dtype=torch.int32, device=device)
 
 
-def attention_units_on_the_matrix_cores(o, device, sizes=(8, 2, 64, 128), n=700, window=100, differential=True, ranges=False):
+def attention_units_on_the_matrix_cores(o, device, sizes=(8, 2, 64, 128), n=700, window=100, differential=True, last=24):
     """`paged_attention_maps_units` (bfloat16, pages of 16 keys) against the plain functions, with the chosen keys of
     `differential_attention_edges`: just inside and just outside the window, at page borders and far back; the
     queries as units of several tokens (a prompt's portion) and as units of one token (decoding), with the keys in
-    one range and cut into several."""
+    one range and cut into several.  last: how many of the last positions are queries (hundreds: the launch has so
+    many units that a wave takes a unit of its own; all of them: a sequence's first tokens are among them)."""
     dtype, page_size = torch.bfloat16, 16
     H, K, dk, dv = sizes
     maps = 2 if differential else 1
@@ -439,8 +440,8 @@ def attention_units_on_the_matrix_cores(o, device, sizes=(8, 2, 64, 128), n=700,
     for win in (window, None):
         kk = keys.clone()
         w_ = win or n
-        rows = list(range(n - 24, n))
-        for i in rows:
+        rows = list(range(n - last, n))
+        for i in rows[-24:]:
             back = [w_ - 1, w_, 1, w_ - 2][i % 4] if win else [n - 30 + i % 3, 400, i % page_size + 1, i][i % 4]
             if i - back >= 0:
                 for h in range(H):

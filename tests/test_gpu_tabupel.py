@@ -53,6 +53,14 @@ def test_attention_units_on_the_matrix_cores(sizes, differential):
     mech.attention_units_on_the_matrix_cores(ops, DEV, sizes=sizes, differential=differential)
 
 
+def test_attention_of_many_units_on_the_matrix_cores():
+    """Launches with thousands of units, as a prompt's portion makes them: a wave takes a unit of its own."""
+    mech.attention_units_on_the_matrix_cores(ops, DEV, sizes=(40, 1, 576, 512), differential=False, last=700)
+    mech.attention_units_on_the_matrix_cores(ops, DEV, sizes=(40, 1, 576, 128), differential=False, last=700)
+    mech.attention_units_on_the_matrix_cores(ops, DEV, sizes=(8, 2, 64, 128), n=2400, differential=True, last=2400)
+    mech.attention_units_on_the_matrix_cores(ops, DEV, sizes=(6, 2, 32, 48), n=1500, window=33, differential=False, last=1400)
+
+
 def test_recurrence_in_portions_and_other_taps():
     mech.recurrence(ops, DEV, torch.float32, cuts=(1, 2, 40, 1, 46))
     mech.recurrence(ops, DEV, torch.bfloat16, T=400, cuts=(100, 1, 129, 64, 2, 104), block=16)
