@@ -147,15 +147,17 @@ def test_long_decoding(tmp_path, dtype):
     cases.long_decoding(tmp_path, DEV, "mixed", dtype, steps=150, page_size=16)
 
 
-@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_recorded_decode_steps(tmp_path, dtype):
+@pytest.mark.parametrize("name, dtype, page_size", [("mixed", "float32", 4), ("mixed", "bfloat16", 4),
+                                                   ("aligned", "bfloat16", 16)])
+def test_recorded_decode_steps(tmp_path, name, dtype, page_size):
     """Decode-only steps are recorded in a HIP graph and replayed: three requests decode together for 40 steps, and
-    each step's logits are those of the same step run eagerly by a second engine (states advance exactly once)."""
-    d = cases.write_model("mixed", str(tmp_path / "m"))
+    each step's logits are those of the same step run eagerly by a second engine (states advance exactly once).  With
+    the aligned sizes in pages of 16 keys the attentions run on the matrix cores, their keys cut into ranges."""
+    d = cases.write_model(name, str(tmp_path / "m"))
     V = plain.load(d)[1]["vocab"]
     prompts = {r: cases.random_tokens(n, V, 70 + n) for r, n in (("a", 9), ("b", 3), ("c", 14))}
     follow = {r: cases.random_tokens(40, V, 90 + len(p)) for r, p in prompts.items()}
-    engines = [cases.make_executor(d, DEV, dtype, page_size=4, num_pages=64, batch=4, max_len=64, graphs=g)
+    engines = [cases.make_executor(d, DEV, dtype, page_size=page_size, num_pages=64, batch=4, max_len=64, graphs=g)
                for g in (True, False)]
     for ex in engines:
         for r, p in prompts.items():
