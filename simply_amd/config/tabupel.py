@@ -180,7 +180,7 @@ class TabupelConfig:
         def norm(name: str) -> PartSpec:
             return PartSpec("rmsnorm", {"dim": D, "eps": self.norm_eps, "scale_plus_one": False}, {"scale": name})
 
-        layers, at = [], {}          # at: config layer -> index among the layers that have tensors of their own
+        layers, at, ignorable = [], {}, []   # at: config layer -> index among the layers that have tensors of their own
         for i, l in enumerate(d["layers"]):
             p, where = f"l{i}.", f"layers[{i}]"
             kind = _get(l, "type", where)
@@ -200,6 +200,8 @@ class TabupelConfig:
                                                "intermediate_size": _positive(_get(mlp, "ff", where + ".mlp", int), "ff")},
                                {"gate_proj": p + "mlp.gate", "up_proj": p + "mlp.up", "down_proj": p + "mlp.down"})
                 norms["pre_ffn"] = norm(p + "norm2")
+            else:
+                ignorable.append(p + "norm2")   # (a folder may hold the norm of a feed-forward that is not there)
             at[i] = len(layers)
             layers.append(LayerSpec(block=PartSpec("pre_norm", {"mult": self.residual_mult}), mixer=self._mixer(i, l),
                                     feed_forward=ffn, norms=norms))
@@ -211,7 +213,8 @@ class TabupelConfig:
             final_norm=norm("final.norm"),
             head=PartSpec("linear_head", {"vocab_size": self.vocab, "dim": D, "soft_cap": float(cap) if cap else None},
                           {"weight": "head"}),
-            max_position=self.max_position, eos_token_ids=self.eos_token_ids, initializer_range=self.initializer_range)
+            max_position=self.max_position, eos_token_ids=self.eos_token_ids, initializer_range=self.initializer_range,
+            ignorable=tuple(ignorable))
         spec.validate()
         return spec
 
