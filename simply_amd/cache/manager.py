@@ -309,11 +309,8 @@ class CacheManager:
         max_blocks = ceil_div(self.max_seq_len, self.page_size)
         for i, (need, cache_from) in enumerate(needs):
             if cache_from is not None:
-                src = self.views[cache_from]
-                if type(src.need) is not type(need) or src.need != need:
-                    raise CacheError(f"schedule entry {i} reads the cache of entry {cache_from}, whose need differs: "
-                                     f"{need} vs {src.need}")
-                self.views.append(self._read_only(src))
+                self.views.append(self._reading_view(i, need, cache_from, by_need, max_blocks, max_step_tokens,
+                                                     group_pages))
                 continue
             self.views.append(self._make_view(i, need, by_need, max_blocks, max_step_tokens, group_pages))
         if device is not None:
@@ -368,6 +365,33 @@ class CacheManager:
         raise CacheError(f"schedule entry {i}: cache need {need!r} says neither page_tensors(...) (something "
                          f"per token) nor slot_tensor(...) (something of fixed size per request), nor is it made "
                          f"of parts that do")
+
+    def _reading_view(self, i: int, need, cache_from: int, by_need, max_blocks, max_step_tokens, group_pages):
+        """The view of schedule entry i, which reads what entry `cache_from` keeps.  A plain need must equal the other
+        entry's and is read as a whole.  Of a need made of parts, what is kept per token (pages) is read from the other
+        entry, part by part in their order, and must equal that entry's; what is of fixed size per request (a state)
+        cannot be shared between layers and is the entry's own."""
+        src = self.views[cache_from]
+        paged = [v for v in self._leaves(src) if v.group_id is not None]
+        if not isinstance(getattr(need, "parts", None), tuple):
+            if type(src.need) is type(need) and src.need == need:
+                return self._read_only(src)
+            for leaf in paged if callable(getattr(need, "page_tensors", None)) else ():
+                if type(leaf.need) is type(need) and leaf.need == need:
+                    return self._read_only(leaf)   # (the pages of an entry that keeps a state beside them)
+            raise CacheError(f"schedule entry {i} reads the cache of entry {cache_from}, whose need differs: "
+                             f"{need} vs {src.need}")
+        view, at = CacheView(need), 0
+        for n in need.parts:
+            if callable(getattr(n, "page_tensors", None)):
+                if at >= len(paged) or type(paged[at].need) is not type(n) or paged[at].need != n:
+                    raise CacheError(f"schedule entry {i} reads the pages of entry {cache_from}, which keeps none like "
+                                     f"{n}")
+                view.parts.append(self._read_only(paged[at]))
+                at += 1
+            else:
+                view.parts.append(self._make_view(i, n, by_need, max_blocks, max_step_tokens, group_pages))
+        return view
 
     @staticmethod
     def _read_only(view: "CacheView") -> "CacheView":

@@ -14,6 +14,7 @@ from .gemma2 import ConfigError, Gemma2Config
 from .zenuzen import ZenuzenConfig
 from .nemidra import NemidraConfig
 from .tabupel import TabupelConfig
+from .rudutar import RudutarConfig
 
 
 def architecture_name(d: Mapping[str, Any]) -> str:
@@ -50,4 +51,4 @@ def load_config(model_dir: str):
 
 
 __all__ = ["EngineConfig", "parse_dtype", "LayerSpec", "ModelSpec", "PartSpec", "ScheduleEntry",
-           "ConfigError", "Gemma2Config", "ZenuzenConfig", "NemidraConfig", "TabupelConfig", "architecture_name", "config_from_dict", "load_config"]
+           "ConfigError", "Gemma2Config", "ZenuzenConfig", "NemidraConfig", "TabupelConfig", "RudutarConfig", "architecture_name", "config_from_dict", "load_config"]

@@ -271,19 +271,21 @@ int paged_attention_generic(const void* q, int dtype, int64_t q_stride, const vo
                             void* out, int64_t out_stride, int T, int H, int Kh, int hd, int page_size, int window,
                             float soft_cap, hipStream_t stream, int hd_v = 0, float scale = 1.f,
                             const void* sinks = nullptr, int sinks_dtype = 0, int maps = 1, int values_in_keys = 0,
-                            int differential = 0, float lambda = 0.f, float eps = 0.f, float mult = 1.f);
+                            int differential = 0, float lambda = 0.f, float eps = 0.f, float mult = 1.f,
+                            const float* slopes = nullptr);
 }  // namespace sa
 
 extern "C" {
 // Attention as sa_paged_attention, for mixers whose values have another size than their keys, whose scores are
 // multiplied by `scale` (before the cap, if there is one) and whose softmax may hold one more term per query head,
 // exp(sinks[h]), that has no key and no value (sinks null: none).  Value pages are [num_pages, Kh, hd_v, page_size];
-// out rows hold H * hd_v elements.
+// out rows hold H * hd_v elements.  slopes (float32 [H], or null): slopes[h] * (query position - key position) is taken
+// off the scaled score.
 int sa_paged_attention_sink(const void* q, int dtype, int64_t q_stride, const void* k_pages, const void* v_pages,
                             const int* block_table, int table_stride, const int* token_seq, const int* positions,
                             void* out, int64_t out_stride, int T, int H, int Kh, int hd, int hd_v, int page_size,
                             int window, float soft_cap, float scale, const void* sinks, int sinks_dtype,
-                            hipStream_t stream);
+                            const float* slopes, hipStream_t stream);
 
 // Attention as sa_paged_attention_sink (no sinks, no cap) with `maps` (1 or 2) score maps per query head: a query row
 // holds H * maps vectors of hd entries (head by head, map by map), a key row maps * hd entries (key pages
@@ -316,10 +318,11 @@ int sa_residual_add_norm(const void* y, int y_dtype, int64_t y_stride, const voi
                          hipStream_t stream);
 
 // out[t, h, :] = (w null ? x[t, h, :] : x[t, h, :] / sqrt(mean(x[t, h, :]^2) + eps) * w) * gate(g[t, h, :]) for H
-// heads of `size` elements; w [size] is shared by the heads; gate 0: sigmoid, 1: silu.  out may be x.
+// heads of `size` elements; w [size] is shared by the heads; gate 0: sigmoid, 1: silu.  out may be x.  gate_per_head: a
+// gate row holds H numbers, one for all entries of a head.
 int sa_gated_heads(const void* x, int x_dtype, int64_t x_stride, const void* g, int g_dtype, int64_t g_stride,
                    const void* w, int w_dtype, float eps, int gate, void* out, int out_dtype, int64_t out_stride, int T,
-                   int H, int size, hipStream_t stream);
+                   int H, int size, int gate_per_head, hipStream_t stream);
 
 // x[t, n] = act(x[t, n]) in place (activation codes of activations.h).
 int sa_activation(void* x, int dtype, int64_t stride, int T, int N, int act, hipStream_t stream);
@@ -458,21 +461,42 @@ int sa_normalized_readout(const float* x, const float* floor, int64_t floor_stri
                           int64_t g_stride, const void* w, int w_dtype, float eps, void* out, int out_dtype,
                           int64_t out_stride, int T, int H, int size, hipStream_t stream);
 
+// ---- what an attention kernel reads, from a fused projection (attention_inputs.hip)
+// A projection row holds [H * dk queries | K * dk keys | K * dv values | ...] (values_are_keys: no value columns, the
+// keys' columns as projected are the values; k_pages null: queries only).  num_taps > 1: every channel passes a causal
+// convolution (taps [channels, num_taps] oldest first; tails float32 [slots, (num_taps - 1) * channels], updated).  norm
+// 0: none; 1: queries and keys head by head with weights [dk]; 2: over the whole row with weights [H * dk] and
+// [K * dk].  Then the first rot_dims entries of every head turn in pairs (i, i + rot_dims / 2) by position *
+// inv_freq[i], and queries are multiplied by 1 + temp_coef * ln(floor((position + 1) / temp_every) + 1) (temp_every 0:
+// not).  Queries go to q_out [T, H * dk], keys and values into their pages.
+int sa_attention_inputs(const void* proj, int dtype, int64_t row_stride, int H, int K, int dk, int dv, int k_at, int v_at,
+                        int values_are_keys, const void* taps, int taps_dtype, int num_taps, float* tails,
+                        int64_t tail_stride, int norm, const void* q_w, const void* k_w, int w_dtype, float eps,
+                        const float* inv_freq, int rot_dims, float temp_coef, int temp_every, const int* seq_meta,
+                        int num_seqs, int max_q_len, const int64_t* slot_mapping, void* q_out, int64_t q_stride,
+                        void* k_pages, void* v_pages, int page_size, hipStream_t stream);
+
 // ---- routed experts (routed.hip)
 // softmax over E logits, the top largest: experts [T, top], weights [T, top] = score * scale.
 int sa_route(const float* logits, int64_t stride, int T, int E, int top, float scale, int* experts, float* weights,
              hipStream_t stream);
+// Scores are sigmoids of the logits.  The choice goes by score + correction[e] (null: by the score); the experts form
+// `groups` equal groups of neighbours, a group's score is the sum of its two largest choice scores, and only experts of
+// the `keep` best groups can be chosen.  weights = score * scale (without the correction, not renormalized).
+int sa_route_choice(const float* logits, int64_t stride, int T, int E, int top, float scale, const void* correction,
+                    int corr_dtype, int groups, int keep, int* experts, float* weights, hipStream_t stream);
 // The most tiles of tile_rows (16 or 64) rows of one expert that P pairs over E experts make.
 int sa_expert_tiles_max(int P, int E, int tile_rows);
 // sorted [P]: the pairs by expert; plan [1 + 2 * sa_expert_tiles_max(P, E, tile_rows)]: the tiles.
 int sa_expert_sort(const int* experts, int P, int E, int tile_rows, int* sorted, int* plan, int plan_words,
                    hipStream_t stream);
-// w2 given: out[row] = act(a . w1[e]^T) * (a . w2[e]^T) in a's type; else out[row] = a . w1[e]^T in 32-bit.  a's row is
+// w2 given: out[row] = act(a . w1[e]^T) * (a . w2[e]^T) in a's type; else out[row] = a . w1[e]^T in 32-bit, or, with
+// `activate`, act(a . w1[e]^T) in a's type (experts without a gate).  a's row is
 // the pair's token (a_by_token) or its place in the sorted order; out's row the pair (out_by_pair) or that place.
 // bfloat16 weights are tiled [E][ceil(N / 16)][ceil(K / 32)][64][8], 32-bit ones row-major [E][N][K].
 int sa_expert_product(const void* a, int dtype, int64_t a_stride, int a_by_token, int top, const void* w1, const void* w2,
                       int N, int K, const int* sorted, const int* plan, int P, int E, int tile_rows, int act, void* out,
-                      int64_t out_stride, int out_by_pair, hipStream_t stream);
+                      int64_t out_stride, int out_by_pair, int activate, hipStream_t stream);
 // out[t] = sum_k weights[t, k] y[t * top + k] + sigmoid(gate[t]) * shared[t]  (shared null: none; gate null: 1).
 int sa_expert_combine(const float* y, const float* weights, int top, const void* shared, int shared_dtype,
                       int64_t shared_stride, const float* gate, int64_t gate_stride, void* out, int out_dtype,

@@ -44,7 +44,7 @@ __global__ __launch_bounds__(kThreads) void paged_attention_generic_kernel(
     const int* __restrict__ block_table, int table_stride, const int* __restrict__ token_seq,
     const int* __restrict__ positions, T* __restrict__ out, int64_t out_stride, int Kh, int G, int hd, int hd_v,
     int page_size, int window, float soft_cap, float scale, const void* __restrict__ sinks, int sinks_dtype,
-    AttentionOptions opt, int G_all) {
+    AttentionOptions opt, int G_all, const float* __restrict__ slopes) {
   // G_all query vectors per key/value head, of which this workgroup takes G (the last one of a head what is left):
   // many heads over one key head need not fit into one workgroup's LDS
   const int gz = blockIdx.z * G;          // the workgroup's first vector among its key head's
@@ -122,6 +122,8 @@ __global__ __launch_bounds__(kThreads) void paged_attention_generic_kernel(
             if (part == 0) {
               s *= scale;
               if (soft_cap > 0.f) s = soft_cap * tanhf(s / soft_cap);
+              // a bias by distance: the head's slope times how far back the key lies is taken off
+              if (slopes != nullptr) s -= slopes[(kh * G_all + gz + g0 + g) / M] * static_cast<float>(pos - (c0 + j));
               s_s[(g0 + g) * kChunk + j] = valid ? s : -INFINITY;
             }
           }
@@ -224,18 +226,18 @@ static void launch_generic(const void* q, int dtype, int64_t q_stride, const voi
                            const int* block_table, int table_stride, const int* token_seq, const int* positions,
                            void* out, int64_t out_stride, int T, int Kh, int G, int hd, int hd_v, int page_size,
                            int window, float soft_cap, float scale, const void* sinks, int sinks_dtype,
-                           AttentionOptions opt, size_t smem, int G_all, hipStream_t stream) {
+                           AttentionOptions opt, size_t smem, int G_all, const float* slopes, hipStream_t stream) {
   const dim3 grid(T, Kh, (G_all + G - 1) / G);
   if (dtype == kF32)
     paged_attention_generic_kernel<float, M><<<grid, kThreads, smem, stream>>>(
         static_cast<const float*>(q), q_stride, static_cast<const float*>(k_pages),
         static_cast<const float*>(v_pages), block_table, table_stride, token_seq, positions, static_cast<float*>(out),
-        out_stride, Kh, G, hd, hd_v, page_size, window, soft_cap, scale, sinks, sinks_dtype, opt, G_all);
+        out_stride, Kh, G, hd, hd_v, page_size, window, soft_cap, scale, sinks, sinks_dtype, opt, G_all, slopes);
   else
     paged_attention_generic_kernel<bf16, M><<<grid, kThreads, smem, stream>>>(
         static_cast<const bf16*>(q), q_stride, static_cast<const bf16*>(k_pages), static_cast<const bf16*>(v_pages),
         block_table, table_stride, token_seq, positions, static_cast<bf16*>(out), out_stride, Kh, G, hd, hd_v, page_size,
-        window, soft_cap, scale, sinks, sinks_dtype, opt, G_all);
+        window, soft_cap, scale, sinks, sinks_dtype, opt, G_all, slopes);
 }
 
 int paged_attention_generic(const void* q, int dtype, int64_t q_stride, const void* k_pages, const void* v_pages,
@@ -243,7 +245,7 @@ int paged_attention_generic(const void* q, int dtype, int64_t q_stride, const vo
                             void* out, int64_t out_stride, int T, int H, int Kh, int hd, int page_size, int window,
                             float soft_cap, hipStream_t stream, int hd_v, float scale, const void* sinks,
                             int sinks_dtype, int maps, int values_in_keys, int differential, float lambda, float eps,
-                            float mult) {
+                            float mult, const float* slopes) {
   int G = H / Kh * maps;   // query vectors per key/value head (below: per workgroup)
   if (hd_v <= 0) hd_v = hd;
   if (maps != 1 && maps != 2) {
@@ -287,11 +289,11 @@ int paged_attention_generic(const void* q, int dtype, int64_t q_stride, const vo
   if (maps == 2)
     launch_generic<2>(q, dtype, q_stride, k_pages, v_pages, block_table, table_stride, token_seq, positions, out,
                       out_stride, T, Kh, G, hd, hd_v, page_size, window, soft_cap, scale, sinks, sinks_dtype, opt, smem,
-                      G_all, stream);
+                      G_all, slopes, stream);
   else
     launch_generic<1>(q, dtype, q_stride, k_pages, v_pages, block_table, table_stride, token_seq, positions, out,
                       out_stride, T, Kh, G, hd, hd_v, page_size, window, soft_cap, scale, sinks, sinks_dtype, opt, smem,
-                      G_all, stream);
+                      G_all, slopes, stream);
   return check_launch("paged_attention_generic");
 }
 

@@ -155,10 +155,11 @@ __device__ inline float gate_value(int kind, float g) {
 __global__ __launch_bounds__(kWave) void gated_heads_kernel(
     const void* __restrict__ x, int x_dtype, int64_t x_stride, const void* __restrict__ g, int g_dtype,
     int64_t g_stride, const void* __restrict__ w, int w_dtype, float eps, int gate, void* __restrict__ out,
-    int out_dtype, int64_t out_stride, int size) {
+    int out_dtype, int64_t out_stride, int size, int gate_per_head) {
+  // gate_per_head: a gate row holds one number per head, which all of the head's entries share
   const int t = blockIdx.x, h = blockIdx.y;
   const size_t xb = static_cast<size_t>(t) * x_stride + static_cast<size_t>(h) * size;
-  const size_t gb = static_cast<size_t>(t) * g_stride + static_cast<size_t>(h) * size;
+  const size_t gb = static_cast<size_t>(t) * g_stride + (gate_per_head ? h : static_cast<size_t>(h) * size);
   const size_t ob = static_cast<size_t>(t) * out_stride + static_cast<size_t>(h) * size;
   float r = 1.f;
   if (w != nullptr) {
@@ -173,7 +174,7 @@ __global__ __launch_bounds__(kWave) void gated_heads_kernel(
   for (int d = threadIdx.x; d < size; d += kWave) {
     float v = load_f(x, x_dtype, xb + d);
     if (w != nullptr) v = v * r * load_f(w, w_dtype, d);
-    store_f(out, out_dtype, ob + d, v * gate_value(gate, load_f(g, g_dtype, gb + d)));
+    store_f(out, out_dtype, ob + d, v * gate_value(gate, load_f(g, g_dtype, gate_per_head ? gb : gb + d)));
   }
 }
 
@@ -420,17 +421,17 @@ extern "C" int sa_residual_add_next_norm(const void* y, int y_dtype, int64_t y_s
 
 extern "C" int sa_gated_heads(const void* x, int x_dtype, int64_t x_stride, const void* g, int g_dtype, int64_t g_stride,
                               const void* w, int w_dtype, float eps, int gate, void* out, int out_dtype,
-                              int64_t out_stride, int T, int H, int size, hipStream_t stream) {
+                              int64_t out_stride, int T, int H, int size, int gate_per_head, hipStream_t stream) {
   if (T == 0) return 0;
   SA_REQUIRE(T > 0 && H > 0 && size > 0 && x != nullptr && g != nullptr && out != nullptr,
              "gated_heads: bad sizes T=%d H=%d size=%d", T, H, size);
   const int64_t width = static_cast<int64_t>(H) * size;
-  SA_REQUIRE(x_stride >= width && g_stride >= width && out_stride >= width, "gated_heads: a row stride is below %lld",
-             (long long)width);
+  SA_REQUIRE(x_stride >= width && g_stride >= (gate_per_head ? H : width) && out_stride >= width,
+             "gated_heads: a row stride is below %lld", (long long)width);
   SA_REQUIRE(gate == 0 || gate == 1, "gated_heads: unknown gate %d (0: sigmoid, 1: silu)", gate);
   SA_REQUIRE(H <= 65535, "gated_heads: at most 65535 heads");
   gated_heads_kernel<<<dim3(T, H), kWave, 0, stream>>>(x, x_dtype, x_stride, g, g_dtype, g_stride, w, w_dtype, eps, gate,
-                                                       out, out_dtype, out_stride, size);
+                                                       out, out_dtype, out_stride, size, gate_per_head);
   return check_launch("gated_heads");
 }
 

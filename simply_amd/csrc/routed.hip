@@ -61,6 +61,91 @@ __global__ __launch_bounds__(kWave) void route_kernel(const float* __restrict__ 
   }
 }
 
+// A wave per token, for routers whose scores are sigmoids of the logits.  The choice is made by score + correction[e]
+// (correction null: by the score); the experts form `groups` equal groups of neighbours, a group's score is the sum of
+// its two largest choice scores (of its only one, in groups of one), and only experts of the `keep` groups with the
+// largest scores can be chosen (of equal ones the lowest index, for groups and for experts).  weight = score * scale,
+// without the correction and not renormalized.  Choice scores can be negative: what is taken or shut out is -inf.
+__global__ __launch_bounds__(kWave) void route_choice_kernel(const float* __restrict__ logits, int64_t stride, int E,
+                                                             int top, float scale, const void* __restrict__ correction,
+                                                             int corr_dtype, int groups, int keep,
+                                                             int* __restrict__ experts, float* __restrict__ weights) {
+  __shared__ float choice_s[kRouteSlots * kWave];
+  __shared__ float group_s[kRouteSlots * kWave];
+  const int t = blockIdx.x, lane = threadIdx.x;
+  float s[kRouteSlots], c[kRouteSlots];
+#pragma unroll
+  for (int i = 0; i < kRouteSlots; ++i) {
+    const int e = lane + i * kWave;
+    s[i] = 0.f;
+    c[i] = -INFINITY;
+    if (e < E) {
+      s[i] = 1.f / (1.f + expf(-logits[static_cast<size_t>(t) * stride + e]));
+      c[i] = correction != nullptr ? s[i] + load_f(correction, corr_dtype, e) : s[i];
+      choice_s[e] = c[i];
+    }
+  }
+  if (groups > 1) {
+    __syncthreads();
+    const int per = E / groups;
+    for (int g = lane; g < groups; g += kWave) {
+      float a = -INFINITY, b = -INFINITY;   // the two largest of the group
+      for (int k = 0; k < per; ++k) {
+        const float v = choice_s[g * per + k];
+        if (v > a) {
+          b = a;
+          a = v;
+        } else if (v > b) {
+          b = v;
+        }
+      }
+      group_s[g] = per > 1 ? a + b : a;
+    }
+    __syncthreads();
+    // the `keep` best groups, one after the other; lane 0 marks them by sign in LDS
+    for (int r = 0; r < keep; ++r) {
+      float best = -INFINITY;
+      for (int g = lane; g < groups; g += kWave) best = fmaxf(best, group_s[g]);
+      best = wave_max(best);
+      float mine = 1e9f;
+      for (int g = lane; g < groups; g += kWave)
+        if (group_s[g] == best && static_cast<float>(g) < mine) mine = static_cast<float>(g);
+      const int g_best = static_cast<int>(-wave_max(-mine));
+      __syncthreads();
+      if (lane == 0) group_s[g_best] = -INFINITY;   // taken: -inf marks a group that stays
+      __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < kRouteSlots; ++i) {
+      const int e = lane + i * kWave;
+      if (e < E && group_s[e / per] != -INFINITY) c[i] = -INFINITY;
+    }
+  }
+  for (int r = 0; r < top; ++r) {
+    float best = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < kRouteSlots; ++i) best = fmaxf(best, c[i]);
+    best = wave_max(best);
+    float mine = 1e9f;
+#pragma unroll
+    for (int i = kRouteSlots - 1; i >= 0; --i)
+      if (c[i] == best && lane + i * kWave < E) mine = static_cast<float>(lane + i * kWave);
+    const int e = static_cast<int>(-wave_max(-mine));
+    float w = 0.f;
+#pragma unroll
+    for (int i = 0; i < kRouteSlots; ++i)
+      if (lane + i * kWave == e) {
+        c[i] = -INFINITY;
+        w = s[i];
+      }
+    w = wave_sum(w);   // (one lane holds it, the others 0)
+    if (lane == 0) {
+      experts[static_cast<size_t>(t) * top + r] = e;
+      weights[static_cast<size_t>(t) * top + r] = w * scale;
+    }
+  }
+}
+
 // One workgroup.  plan: [0] number of tiles; [1 .. 1 + 2 * max_tiles): per tile its expert and its first row in the
 // sorted order with the number of its rows packed as first * 128 + rows.  sorted [P]: pair indices by expert.
 __global__ __launch_bounds__(1024) void sort_kernel(const int* __restrict__ experts, int P, int E,
@@ -120,7 +205,8 @@ template <typename T, bool GATED, int RT>
 __global__ __launch_bounds__(256) void expert_product_kernel(
     const T* __restrict__ a, int64_t a_stride, int a_by_token, int top, const T* __restrict__ w1, const T* __restrict__ w2,
     int N, int K, const int* __restrict__ sorted, const int* __restrict__ plan, int act, void* __restrict__ out,
-    int64_t out_stride, int out_by_pair) {
+    int64_t out_stride, int out_by_pair, int activate) {
+  // activate (without a second weight): out[row] = act(a . w1[e]^T) in a's type instead of the 32-bit product
   const int tile = blockIdx.x;
   if (tile >= plan[0]) return;
   const int e = plan[1 + 2 * tile], packed = plan[2 + 2 * tile];
@@ -202,6 +288,8 @@ __global__ __launch_bounds__(256) void expert_product_kernel(
         if constexpr (GATED) {
           const float v = gated_activation(act, to_float(float_to_bf16(accg[s][i]))) * to_float(float_to_bf16(accu[s][i]));
           static_cast<bf16*>(out)[orow + n] = float_to_bf16(v);
+        } else if (activate) {
+          static_cast<bf16*>(out)[orow + n] = float_to_bf16(gated_activation(act, to_float(float_to_bf16(accg[s][i]))));
         } else {
           static_cast<float*>(out)[orow + n] = accg[s][i];
         }
@@ -223,7 +311,7 @@ __global__ __launch_bounds__(256) void expert_product_kernel(
         for (int k = 0; k < K; ++k) su = fmaf(to_float(arow[k]), to_float(u[k]), su);
         static_cast<float*>(out)[orow + n] = gated_activation_exact(act, sg) * su;
       } else {
-        static_cast<float*>(out)[orow + n] = sg;
+        static_cast<float*>(out)[orow + n] = activate ? gated_activation_exact(act, sg) : sg;
       }
     }
   }
@@ -239,7 +327,7 @@ template <bool GATED>
 __global__ __launch_bounds__(256) void expert_product_rows64_kernel(
     const bf16* __restrict__ a, int64_t a_stride, int a_by_token, int top, const bf16* __restrict__ w1,
     const bf16* __restrict__ w2, int N, int K, const int* __restrict__ sorted, const int* __restrict__ plan, int act,
-    void* __restrict__ out, int64_t out_stride, int out_by_pair) {
+    void* __restrict__ out, int64_t out_stride, int out_by_pair, int activate) {
   __shared__ bf16x8 rows_lds[4][kChunkK / 32][kWave];   // [sub-tile of 16 rows][k tile of the chunk][lane]
   __shared__ int pair_of[kTileRowsMax];
   const int tile = blockIdx.x;
@@ -334,6 +422,9 @@ __global__ __launch_bounds__(256) void expert_product_rows64_kernel(
         if constexpr (GATED) {
           const float v = gated_activation(act, to_float(float_to_bf16(accg[s][j][i]))) * to_float(float_to_bf16(accu[s][j][i]));
           static_cast<bf16*>(out)[orow + n] = float_to_bf16(v);
+        } else if (activate) {
+          static_cast<bf16*>(out)[orow + n] =
+              float_to_bf16(gated_activation(act, to_float(float_to_bf16(accg[s][j][i]))));
         } else {
           static_cast<float*>(out)[orow + n] = accg[s][j][i];
         }
@@ -372,6 +463,23 @@ extern "C" int sa_route(const float* logits, int64_t stride, int T, int E, int t
   return check_launch("route");
 }
 
+extern "C" int sa_route_choice(const float* logits, int64_t stride, int T, int E, int top, float scale,
+                               const void* correction, int corr_dtype, int groups, int keep, int* experts,
+                               float* weights, hipStream_t stream) {
+  if (T == 0) return 0;
+  SA_REQUIRE(T > 0 && E > 0 && E <= kRouteSlots * kWave && top > 0 && stride >= E,
+             "route_choice: bad sizes T=%d E=%d top=%d (at most %d experts)", T, E, top, kRouteSlots * kWave);
+  SA_REQUIRE(groups >= 1 && E % groups == 0 && keep >= 1 && keep <= groups,
+             "route_choice: %d experts in %d groups of which %d stay", E, groups, keep);
+  SA_REQUIRE(top <= keep * (E / groups), "route_choice: %d experts cannot be chosen from %d groups of %d", top, keep,
+             E / groups);
+  SA_REQUIRE(correction == nullptr || corr_dtype == kF32 || corr_dtype == kBF16, "route_choice: unknown dtype %d",
+             corr_dtype);
+  route_choice_kernel<<<T, kWave, 0, stream>>>(logits, stride, E, top, scale, correction, corr_dtype, groups, keep,
+                                               experts, weights);
+  return check_launch("route_choice");
+}
+
 extern "C" int sa_expert_tiles_max(int P, int E, int tile_rows) {
   return (P + tile_rows - 1) / tile_rows + (E < P ? E : P);
 }
@@ -391,9 +499,10 @@ extern "C" int sa_expert_sort(const int* experts, int P, int E, int tile_rows, i
 
 extern "C" int sa_expert_product(const void* a, int dtype, int64_t a_stride, int a_by_token, int top, const void* w1,
                                  const void* w2, int N, int K, const int* sorted, const int* plan, int P, int E,
-                                 int tile_rows, int act, void* out, int64_t out_stride, int out_by_pair,
+                                 int tile_rows, int act, void* out, int64_t out_stride, int out_by_pair, int activate,
                                  hipStream_t stream) {
   if (P == 0) return 0;
+  SA_REQUIRE(!activate || w2 == nullptr, "expert_product: a gated product has its activation already");
   SA_REQUIRE(P > 0 && E > 0 && N > 0 && K > 0 && top > 0 && a_stride >= K && out_stride >= N,
              "expert_product: bad sizes P=%d E=%d N=%d K=%d", P, E, N, K);
   SA_REQUIRE(a != nullptr && w1 != nullptr && sorted != nullptr && plan != nullptr && out != nullptr,
@@ -407,7 +516,8 @@ extern "C" int sa_expert_product(const void* a, int dtype, int64_t a_stride, int
 #define SA_EXPERT(T, G, RT)                                                                                            \
   expert_product_kernel<T, G, RT><<<grid, 256, 0, stream>>>(static_cast<const T*>(a), a_stride, a_by_token, top,        \
                                                              static_cast<const T*>(w1), static_cast<const T*>(w2), N,  \
-                                                             K, sorted, plan, act, out, out_stride, out_by_pair)
+                                                             K, sorted, plan, act, out, out_stride, out_by_pair,       \
+                                                             activate)
   if (dtype == kBF16) {
     if (tile_rows == 16) {
       if (gated) SA_EXPERT(bf16, true, 1);
@@ -417,11 +527,11 @@ extern "C" int sa_expert_product(const void* a, int dtype, int64_t a_stride, int
       if (gated)
         expert_product_rows64_kernel<true><<<wide, 256, 0, stream>>>(
             static_cast<const bf16*>(a), a_stride, a_by_token, top, static_cast<const bf16*>(w1),
-            static_cast<const bf16*>(w2), N, K, sorted, plan, act, out, out_stride, out_by_pair);
+            static_cast<const bf16*>(w2), N, K, sorted, plan, act, out, out_stride, out_by_pair, 0);
       else
         expert_product_rows64_kernel<false><<<wide, 256, 0, stream>>>(
             static_cast<const bf16*>(a), a_stride, a_by_token, top, static_cast<const bf16*>(w1), nullptr, N, K, sorted,
-            plan, act, out, out_stride, out_by_pair);
+            plan, act, out, out_stride, out_by_pair, activate);
     }
   } else {
     if (gated) SA_EXPERT(float, true, 1);

@@ -178,7 +178,8 @@ extern "C" int sa_paged_attention_sink(const void* q, int dtype, int64_t q_strid
                                        const void* v_pages, const int* block_table, int table_stride,
                                        const int* token_seq, const int* positions, void* out, int64_t out_stride, int T,
                                        int H, int Kh, int hd, int hd_v, int page_size, int window, float soft_cap,
-                                       float scale, const void* sinks, int sinks_dtype, hipStream_t stream) {
+                                       float scale, const void* sinks, int sinks_dtype, const float* slopes,
+                                       hipStream_t stream) {
   if (T == 0) return 0;
   SA_REQUIRE(dtype == kF32 || dtype == kBF16, "paged_attention_sink: unknown dtype %d", dtype);
   SA_REQUIRE(T > 0 && H > 0 && Kh > 0 && hd > 0 && hd_v > 0 && page_size > 0,
@@ -190,7 +191,7 @@ extern "C" int sa_paged_attention_sink(const void* q, int dtype, int64_t q_strid
   SA_REQUIRE(sinks == nullptr || sinks_dtype == kF32 || sinks_dtype == kBF16, "paged_attention_sink: unknown sink dtype");
   return paged_attention_generic(q, dtype, q_stride, k_pages, v_pages, block_table, table_stride, token_seq, positions,
                                  out, out_stride, T, H, Kh, hd, page_size, window, soft_cap, stream, hd_v, scale, sinks,
-                                 sinks_dtype);
+                                 sinks_dtype, 1, 0, 0, 0.f, 0.f, 1.f, slopes);
 }
 
 extern "C" int sa_paged_attention_maps(const void* q, int dtype, int64_t q_stride, const void* k_pages,

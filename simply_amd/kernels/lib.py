@@ -55,9 +55,10 @@ _SIGNATURES = {
     "sa_score": [_P, _L, _I, _I, _P, _P, _P, _P, _P, _P],
     "sa_probe_hbm_read": [_P, _L, _P, _P, _P],
     "sa_probe_mfma": [_P, _I, _I, _P, _P],
-    "sa_paged_attention_sink": [_P, _I, _L, _P, _P, _P, _I, _P, _P, _P, _L, _I, _I, _I, _I, _I, _I, _I, _F, _F, _P, _I, _P],
+    "sa_paged_attention_sink": [_P, _I, _L, _P, _P, _P, _I, _P, _P, _P, _L, _I, _I, _I, _I, _I, _I, _I, _F, _F, _P, _I, _P,
+                                _P],
     "sa_residual_add_norm": [_P, _I, _L, _P, _I, _F, _I, _F, _P, _P, _I, _I, _I, _P],
-    "sa_gated_heads": [_P, _I, _L, _P, _I, _L, _P, _I, _F, _I, _P, _I, _L, _I, _I, _I, _P],
+    "sa_gated_heads": [_P, _I, _L, _P, _I, _L, _P, _I, _F, _I, _P, _I, _L, _I, _I, _I, _I, _P],
     "sa_activation": [_P, _I, _L, _I, _I, _I, _P],
     "sa_qk_norm_rope_cache_write": [_P, _I, _L, _P, _P, _I, _F, _F, _P, _L, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
     "sa_paged_attention_decode_sink": [_P, _L, _P, _P, _P, _I, _P, _I, _I, _P, _L, _I, _I, _I, _I, _I, _F, _I, _I, _I, _P,
@@ -90,7 +91,10 @@ _SIGNATURES = {
     "sa_normalized_readout": [_P, _P, _L, _P, _I, _L, _P, _I, _F, _P, _I, _L, _I, _I, _I, _P],
     "sa_route": [_P, _L, _I, _I, _I, _F, _P, _P, _P],
     "sa_expert_sort": [_P, _I, _I, _I, _P, _P, _I, _P],
-    "sa_expert_product": [_P, _I, _L, _I, _I, _P, _P, _I, _I, _P, _P, _I, _I, _I, _I, _P, _L, _I, _P],
+    "sa_expert_product": [_P, _I, _L, _I, _I, _P, _P, _I, _I, _P, _P, _I, _I, _I, _I, _P, _L, _I, _I, _P],
+    "sa_route_choice": [_P, _L, _I, _I, _I, _F, _P, _I, _I, _I, _P, _P, _P],
+    "sa_attention_inputs": [_P, _I, _L, _I, _I, _I, _I, _I, _I, _I, _P, _I, _I, _P, _L, _I, _P, _P, _I, _F, _P, _I, _F, _I,
+                            _P, _I, _I, _P, _P, _L, _P, _P, _I, _P],
     "sa_expert_combine": [_P, _P, _I, _P, _I, _L, _P, _L, _P, _I, _L, _I, _I, _P],
     "sa_sample": [_P, _L, _I, _I, _P, _P, _P, _P, _P, _P, _P, _I, _P, _L, _P],
 }

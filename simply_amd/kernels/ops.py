@@ -691,11 +691,14 @@ def paged_attention_prefill(q: torch.Tensor, k_pages: torch.Tensor, v_pages: tor
 def paged_attention_sink(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,
                          token_seq: torch.Tensor, positions: torch.Tensor, num_heads: int, *, scale: float = 1.0,
                          sinks: torch.Tensor | None = None, window: int | None = None, soft_cap: float | None = None,
-                         out: torch.Tensor | None = None) -> torch.Tensor:
+                         out: torch.Tensor | None = None, slopes: torch.Tensor | None = None) -> torch.Tensor:
     """Attention whose values may have another size than its keys (key pages [pages, K, P, dk], value pages
     [pages, K, dv, P]), with scores times `scale` and, if `sinks` [H] is given, one more term exp(sinks[h]) in every
-    softmax sum that has no value.  q: [T, >= H * dk] rows.  Returns [T, H * dv]."""
-    _dev(q, k_pages, v_pages, block_table, token_seq, positions, sinks, out)
+    softmax sum that has no value.  slopes (float32 [H]): slopes[h] * (query position - key position) is taken off
+    the scaled scores.  q: [T, >= H * dk] rows.  Returns [T, H * dv]."""
+    _dev(q, k_pages, v_pages, block_table, token_seq, positions, sinks, out, slopes)
+    if slopes is not None and (slopes.dtype != torch.float32 or slopes.numel() != num_heads or not slopes.is_contiguous()):
+        raise KernelError("paged_attention_sink: slopes must be contiguous float32, one per query head")
     q_stride = _rows(q, "paged_attention_sink: q")
     T = q.shape[0]
     if k_pages.dim() != 4 or v_pages.dim() != 4 or not k_pages.is_contiguous() or not v_pages.is_contiguous() \
@@ -722,7 +725,7 @@ def paged_attention_sink(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.
     _lib.call("sa_paged_attention_sink", _ptr(q), _code(q), q_stride, _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
               block_table.stride(0), _ptr(token_seq), _ptr(positions), _ptr(out), out_stride, T, num_heads, Kh, dk, dv,
               page_size, int(window or 0), float(soft_cap or 0.0), float(scale), _ptr(sinks),
-              _code(sinks) if sinks is not None else 0, _stream())
+              _code(sinks) if sinks is not None else 0, _ptr(slopes), _stream())
     return out
 
 
@@ -902,15 +905,15 @@ GATE_SIGMOID, GATE_SILU = 0, 1
 
 def gated_heads(x: torch.Tensor, gate: torch.Tensor, num_heads: int, size: int, *, kind: int,
                 weight: torch.Tensor | None = None, eps: float = 0.0, out_dtype: torch.dtype | None = None,
-                out: torch.Tensor | None = None) -> torch.Tensor:
+                out: torch.Tensor | None = None, per_head: bool = False) -> torch.Tensor:
     """out[t, h] = (x[t, h] normed over the head's `size` entries and times weight [size], if a weight is given,
     else x[t, h]) * sigmoid(gate[t, h]) or * silu(gate[t, h]).  x, gate: rows of num_heads * size (views with a
-    row stride are fine)."""
+    row stride are fine); per_head: gate rows of num_heads, one number for all entries of a head."""
     _dev(x, gate, weight, out)
     T = x.shape[0]
     width = num_heads * size
     xs, gs = _rows(x, "gated_heads: x"), _rows(gate, "gated_heads: gate")
-    if x.shape[1] != width or tuple(gate.shape) != (T, width):
+    if x.shape[1] != width or tuple(gate.shape) != (T, num_heads if per_head else width):
         raise KernelError(f"gated_heads: rows of {width} expected, got x {tuple(x.shape)} gate {tuple(gate.shape)}")
     if weight is not None and (weight.numel() != size or not weight.is_contiguous()):
         raise KernelError("gated_heads: the norm weight has one entry per element of a head")
@@ -923,7 +926,7 @@ def gated_heads(x: torch.Tensor, gate: torch.Tensor, num_heads: int, size: int, 
     os_ = _rows(out, "gated_heads: out")
     _lib.call("sa_gated_heads", _ptr(x), _code(x), xs, _ptr(gate), _code(gate), gs, _ptr(weight),
               _code(weight) if weight is not None else 0, float(eps), int(kind), _ptr(out), _code(out), os_, T,
-              num_heads, size, _stream())
+              num_heads, size, int(bool(per_head)), _stream())
     return out
 
 
@@ -980,6 +983,76 @@ def qk_norm_rope_cache_write(proj: torch.Tensor, positions: torch.Tensor, inv_fr
               _code(v_mix) if v_mix is not None else 0, _ptr(slot_mapping), _ptr(k_pages), _ptr(v_pages), T, H, K, dk,
               dv, int(page_size), _stream())
     return proj
+
+
+def attention_inputs(proj: torch.Tensor, seq_meta: torch.Tensor, num_seqs: int, max_q_len: int, num_heads: int,
+                     num_kv_heads: int, key_dim: int, value_dim: int, *, values_are_keys: bool = False,
+                     taps: torch.Tensor | None = None, tails: torch.Tensor | None = None, norm: str | None = None,
+                     q_weight: torch.Tensor | None = None, k_weight: torch.Tensor | None = None, eps: float = 0.0,
+                     inv_freq: torch.Tensor | None = None, rot_dims: int = 0, temp_coef: float = 0.0, temp_every: int = 0,
+                     slot_mapping: torch.Tensor | None = None, k_pages: torch.Tensor | None = None,
+                     v_pages: torch.Tensor | None = None) -> torch.Tensor:
+    """From fused projection rows [H * dk queries | K * dk keys | K * dv values | ...] of a ragged step (seq_meta) to
+    what an attention kernel reads.  taps [channels, n] with tails float32 [slots, (n - 1) * channels]: every channel
+    passes a causal convolution first (taps oldest first; the tails are the rows that earlier steps projected last and
+    are brought up to date).  norm 'head': queries and keys divided by each head's root mean square, times q_weight /
+    k_weight [dk]; 'row': by the whole row's, times weights [H * dk] / [K * dk].  Then the first rot_dims entries of
+    every head turn in pairs (i, i + rot_dims / 2) by position * inv_freq[i]; queries are multiplied by
+    1 + temp_coef * ln(floor((position + 1) / temp_every) + 1) (temp_every 0: not).  Keys go into k_pages, values
+    (values_are_keys: the keys' columns as projected, and there are no value columns) into v_pages; without pages the
+    rows hold queries only.  Returns the queries [T, H * dk] in proj's type."""
+    _dev(proj, seq_meta, taps, tails, q_weight, k_weight, inv_freq, slot_mapping, k_pages, v_pages)
+    stride = _rows(proj, "attention_inputs: proj")
+    T = proj.shape[0]
+    H, K, dk, dv = int(num_heads), int(num_kv_heads), int(key_dim), int(value_dim)
+    _seq_meta(seq_meta, num_seqs, "attention_inputs")
+    own = k_pages is not None
+    C = (H + K) * dk + (0 if values_are_keys else K * dv) if own else H * dk
+    if proj.shape[1] < C:
+        raise KernelError(f"attention_inputs: rows of {proj.shape[1]} are shorter than the {C} columns")
+    code = {None: 0, "head": 1, "row": 2}.get(norm)
+    if code is None:
+        raise KernelError(f"attention_inputs: norm is None, 'head' or 'row', not {norm!r}")
+    w_dtype = None
+    if code:
+        wanted = [(q_weight, dk if code == 1 else H * dk)] + ([(k_weight, dk if code == 1 else K * dk)] if own else [])
+        for w, n in wanted:
+            if w is None or not w.is_contiguous() or w.numel() != n or (w_dtype is not None and w.dtype != w_dtype):
+                raise KernelError("attention_inputs: norm weights are contiguous, of one type, one entry per normed entry")
+            w_dtype = w.dtype
+    n_taps = 0
+    if taps is not None:
+        if taps.dim() != 2 or taps.shape[0] != C or not taps.is_contiguous():
+            raise KernelError(f"attention_inputs: taps {tuple(taps.shape)} for {C} channels")
+        n_taps = taps.shape[1]
+        if n_taps > 1 and (tails is None or tails.dtype != torch.float32 or tails.dim() != 2 or tails.stride(1) != 1
+                           or tails.shape[1] < (n_taps - 1) * C):
+            raise KernelError("attention_inputs: tails must be float32 [slots, >= (taps - 1) * channels]")
+    if rot_dims and (inv_freq is None or inv_freq.dtype != torch.float32 or inv_freq.numel() != rot_dims // 2
+                     or not inv_freq.is_contiguous() or rot_dims % 2 or rot_dims > dk):
+        raise KernelError("attention_inputs: inv_freq must be float32 [rot_dims / 2], rot_dims even, <= dk")
+    page_size = 1
+    if own:
+        if v_pages is None or slot_mapping is None:
+            raise KernelError("attention_inputs: key pages, value pages and slots come together")
+        if k_pages.dim() != 4 or v_pages.dim() != 4 or not k_pages.is_contiguous() or not v_pages.is_contiguous() \
+                or k_pages.dtype != proj.dtype or v_pages.dtype != proj.dtype:
+            raise KernelError(f"attention_inputs: pages must be contiguous 4-D tensors of {proj.dtype}")
+        n, _, page_size, _ = k_pages.shape
+        if tuple(k_pages.shape) != (n, K, page_size, dk) or tuple(v_pages.shape) != (n, K, dv, page_size):
+            raise KernelError(f"attention_inputs: pages {tuple(k_pages.shape)}, {tuple(v_pages.shape)} do not match "
+                              f"{K} heads of key size {dk} and value size {dv}")
+        if slot_mapping.dtype != torch.int64 or slot_mapping.numel() < T or not slot_mapping.is_contiguous():
+            raise KernelError("attention_inputs: slot_mapping must be int64 [T]")
+    q_out = torch.empty((T, H * dk), dtype=proj.dtype, device=proj.device)
+    _lib.call("sa_attention_inputs", _ptr(proj), _code(proj), stride, H, K, dk, dv, H * dk, (H + K) * dk,
+              int(bool(values_are_keys)), _ptr(taps), _code(taps) if taps is not None else 0, int(n_taps),
+              _ptr(tails) if n_taps > 1 else None, tails.stride(0) if n_taps > 1 else 0, code, _ptr(q_weight),
+              _ptr(k_weight) if own else None, _CODES[w_dtype] if w_dtype is not None else 0, float(eps), _ptr(inv_freq),
+              int(rot_dims), float(temp_coef), int(temp_every), _ptr(seq_meta), int(num_seqs), int(max_q_len),
+              _ptr(slot_mapping) if own else None, _ptr(q_out), q_out.stride(0), _ptr(k_pages), _ptr(v_pages) if own else None,
+              int(page_size), _stream())
+    return q_out
 
 
 # --------------------------------------------------------------------------- recurrent mixers
@@ -1485,18 +1558,40 @@ def route(logits: torch.Tensor, top: int, scale: float) -> tuple[torch.Tensor, t
     return experts, weights
 
 
+def route_choice(logits: torch.Tensor, top: int, scale: float, *, correction: torch.Tensor | None = None,
+                 groups: int = 1, keep: int = 1) -> tuple[torch.Tensor, torch.Tensor]:
+    """Scores are sigmoids of the logits (float32 [T, E]); the `top` experts with the largest score + correction[e] are
+    chosen, among the `keep` groups (of `groups` equal groups of neighbouring experts) whose two largest choice scores
+    have the largest sums.  Returns (experts int32 [T, top], weights float32 [T, top] = score * scale, the score
+    without the correction), largest choice first."""
+    _dev(logits, correction)
+    T, E = logits.shape
+    if logits.dtype != torch.float32:
+        raise KernelError("route_choice: the router's logits are float32")
+    if correction is not None and (correction.numel() != E or not correction.is_contiguous()):
+        raise KernelError(f"route_choice: a correction of {correction.numel()} entries for {E} experts")
+    experts = torch.empty((T, top), dtype=torch.int32, device=logits.device)
+    weights = torch.empty((T, top), dtype=torch.float32, device=logits.device)
+    _lib.call("sa_route_choice", _ptr(logits), _rows(logits, "route_choice: logits"), T, E, int(top), float(scale),
+              _ptr(correction), _code(correction) if correction is not None else 0, int(groups), int(keep),
+              _ptr(experts), _ptr(weights), _stream())
+    return experts, weights
+
+
 def routed_experts(x: torch.Tensor, experts: torch.Tensor, weights: torch.Tensor, gate_w, up_w, down_w, activation: int,
                    *, shared: torch.Tensor | None = None, shared_gate: torch.Tensor | None = None,
                    out_dtype: torch.dtype | None = None) -> torch.Tensor:
     """sum_k weights[t, k] * down[e](act(gate[e] x) * (up[e] x)) with e = experts[t, k], plus sigmoid(shared_gate[t]) *
     shared[t] (shared None: nothing; shared_gate None: shared as it is).  gate_w, up_w, down_w: `packing.ExpertStack`s
-    (every expert's matrix, tiled if bfloat16).  x [T, D] in the weights' type; shared_gate float32 [T, 1]."""
-    _dev(x, experts, weights, gate_w.data, up_w.data, down_w.data, shared, shared_gate)
+    (every expert's matrix, tiled if bfloat16).  x [T, D] in the weights' type; shared_gate float32 [T, 1].
+    gate_w None: experts without a gate, down[e](act(up[e] x))."""
+    _dev(x, experts, weights, gate_w.data if gate_w is not None else None, up_w.data, down_w.data, shared, shared_gate)
     T, D = x.shape
-    top, E, F = experts.shape[1], gate_w.experts, gate_w.rows
-    if (up_w.experts, up_w.rows, up_w.cols) != (E, F, D) or gate_w.cols != D or (down_w.experts, down_w.rows, down_w.cols) != (E, D, F):
+    top, E, F = experts.shape[1], up_w.experts, up_w.rows
+    if up_w.cols != D or (gate_w is not None and (gate_w.experts, gate_w.rows, gate_w.cols) != (E, F, D)) \
+            or (down_w.experts, down_w.rows, down_w.cols) != (E, D, F):
         raise KernelError("routed_experts: the experts' matrices do not go together")
-    if x.dtype != gate_w.data.dtype or gate_w.tiled != (x.dtype == torch.bfloat16):
+    if x.dtype != up_w.data.dtype or up_w.tiled != (x.dtype == torch.bfloat16):
         raise KernelError("routed_experts: bfloat16 rows go with tiled weights, float32 rows with row-major ones")
     if experts.dtype != torch.int32 or not experts.is_contiguous() or tuple(weights.shape) != (T, top) \
             or weights.dtype != torch.float32 or not weights.is_contiguous():
@@ -1510,11 +1605,13 @@ def routed_experts(x: torch.Tensor, experts: torch.Tensor, weights: torch.Tensor
     plan = torch.empty(1 + 2 * max_tiles, dtype=torch.int32, device=dev)
     _lib.call("sa_expert_sort", _ptr(experts), P, E, tile_rows, _ptr(sorted_), _ptr(plan), plan.numel(), _stream())
     h = torch.empty((P, F), dtype=x.dtype, device=dev)
-    _lib.call("sa_expert_product", _ptr(x), _code(x), _rows(x, "routed_experts: x"), 1, top, _ptr(gate_w.data),
-              _ptr(up_w.data), F, D, _ptr(sorted_), _ptr(plan), P, E, tile_rows, int(activation), _ptr(h), F, 0, _stream())
+    first, second = (gate_w.data, up_w.data) if gate_w is not None else (up_w.data, None)
+    _lib.call("sa_expert_product", _ptr(x), _code(x), _rows(x, "routed_experts: x"), 1, top, _ptr(first),
+              _ptr(second), F, D, _ptr(sorted_), _ptr(plan), P, E, tile_rows, int(activation), _ptr(h), F, 0,
+              int(gate_w is None), _stream())
     y = torch.empty((P, D), dtype=torch.float32, device=dev)
     _lib.call("sa_expert_product", _ptr(h), _code(h), F, 0, top, _ptr(down_w.data), None, D, F, _ptr(sorted_), _ptr(plan), P,
-              E, tile_rows, 0, _ptr(y), D, 1, _stream())
+              E, tile_rows, 0, _ptr(y), D, 1, 0, _stream())
     out = torch.empty((T, D), dtype=out_dtype or x.dtype, device=dev)
     if shared is not None and tuple(shared.shape) != (T, D):
         raise KernelError("routed_experts: the shared expert's rows do not match")

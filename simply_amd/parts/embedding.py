@@ -33,6 +33,28 @@ class ScaledEmbedding(Part):
         return ops.embed(self.table, tokens, scale)
 
 
+@EMBEDDINGS.register("normed_embedding")
+class NormedEmbedding(Part):
+    """The token's row divided by its root mean square (eps inside the root) and multiplied by a weight (`plus_one`:
+    by one plus the weight): a norm on the embedding before the first layer."""
+
+    def __init__(self, vocab_size: int, dim: int, eps: float, plus_one: bool = False):
+        self.vocab_size, self.dim, self.eps, self.plus_one = int(vocab_size), int(dim), float(eps), bool(plus_one)
+        self.table = self.norm = None
+
+    def param_specs(self):
+        return {"table": ParamSpec((self.vocab_size, self.dim), role="matrix", init="weight"),
+                "norm": ParamSpec((self.dim,), role="vector", init="norm")}
+
+    def load(self, tensors):
+        self.table = as_product_weight(tensors["table"], shared=True)
+        self.norm = tensors["norm"].contiguous()
+
+    def forward(self, tokens: torch.Tensor) -> torch.Tensor:
+        """tokens int32 [T] -> float32 residual stream [T, D]."""
+        return ops.rmsnorm(ops.embed(self.table, tokens, 1.0), self.norm, self.eps, self.plus_one, torch.float32)
+
+
 @EMBEDDINGS.register("summed_embedding")
 class SummedEmbedding(Part):
     """The token's row, plus (with `pair_buckets`) a row for the pair of the token and the one before it, chosen by

@@ -80,28 +80,52 @@ class GatedDense(FeedForward):
 
 @FEED_FORWARDS.register("routed_experts")
 class RoutedExperts(FeedForward):
-    """A mixture of experts: `num_experts` gated feed-forwards without biases, down(act(gate x) * (up x)), of which every
-    token uses the `top` ones with the largest router scores.  Scores are the softmax of the router's logits over all
-    experts (32-bit); an expert's result is weighted by its score times `router_scale`, the weights are not renormalized.
-    With `shared_size`, one more such feed-forward runs for every token and is added, times sigmoid(w . x) (one
-    number per token) if `shared_gate`."""
+    """A mixture of experts: `num_experts` feed-forwards without biases, of which every token uses the `top` ones that
+    the router chooses; an expert's result is weighted by its score times `router_scale`, the weights are not
+    renormalized.
+
+      gated       True: an expert is down(act(gate x) * (up x)); False: down(act(up x)), and there are no gate tensors
+      router      'softmax': scores are the softmax of the router's logits over all experts (32-bit), the largest are
+                  chosen; 'sigmoid': scores are sigmoids of the logits, the choice goes by score + a stored correction
+                  per expert (`correction`) among the experts of the `keep_groups` best of `num_groups` equal groups of
+                  neighbours (a group's score: the sum of its two largest choice scores), and the weights are the
+                  scores without the correction
+      shared_size one more feed-forward of the experts' form runs for every token and is added, times sigmoid(w . x)
+                  (one number per token) if `shared_gate`."""
 
     def __init__(self, hidden_size: int, num_experts: int, top: int, expert_size: int, router_scale: float = 1.0,
-                 activation: str = "silu", shared_size: int | None = None, shared_gate: bool = True):
+                 activation: str = "silu", shared_size: int | None = None, shared_gate: bool = True, gated: bool = True,
+                 router: str = "softmax", correction: bool = False, num_groups: int = 1, keep_groups: int = 1):
         self.hidden_size, self.num_experts, self.top = int(hidden_size), int(num_experts), int(top)
         self.expert_size, self.router_scale = int(expert_size), float(router_scale)
         if not 1 <= self.top <= self.num_experts:
             raise ValueError(f"routed_experts: top {top} of {num_experts} experts")
+        if router not in ("softmax", "sigmoid"):
+            raise ValueError(f"routed_experts: the router is 'softmax' or 'sigmoid', not {router!r}")
+        self.router_kind, self.correction = router, bool(correction)
+        self.num_groups, self.keep_groups = int(num_groups), int(keep_groups)
+        if router == "softmax" and (self.correction or self.num_groups != 1):
+            raise ValueError("routed_experts: a correction and groups go with the sigmoid router")
+        if self.num_groups < 1 or self.num_experts % self.num_groups or not 1 <= self.keep_groups <= self.num_groups \
+                or self.top > self.keep_groups * (self.num_experts // self.num_groups):
+            raise ValueError(f"routed_experts: {num_experts} experts in {num_groups} groups of which {keep_groups} stay "
+                             f"do not give {top} choices")
+        self.gated = bool(gated)
         self.activation_code = int(ACTIVATIONS.get(activation))
-        self.shared = GatedDense(hidden_size, int(shared_size), activation) if shared_size else None
+        shared_cls = GatedDense if self.gated else Dense
+        self.shared = shared_cls(hidden_size, int(shared_size), activation) if shared_size else None
         self.shared_gate = bool(shared_gate) and self.shared is not None
-        self.router = self.gate_w = self.up_w = self.down_w = None
+        self.router = self.gate_w = self.up_w = self.down_w = self.correction_w = None
 
     def param_specs(self):
         D, F, E = self.hidden_size, self.expert_size, self.num_experts
         specs = {"router": ParamSpec((E, D))}
+        if self.correction:
+            specs["correction"] = ParamSpec((E,), role="vector", init="norm")
         for e in range(E):
-            specs.update({f"e{e}.gate": ParamSpec((F, D)), f"e{e}.up": ParamSpec((F, D)), f"e{e}.down": ParamSpec((D, F))})
+            if self.gated:
+                specs[f"e{e}.gate"] = ParamSpec((F, D))
+            specs.update({f"e{e}.up": ParamSpec((F, D)), f"e{e}.down": ParamSpec((D, F))})
         if self.shared is not None:
             specs.update({"shared." + n: s for n, s in self.shared.param_specs().items()})
             if self.shared_gate:
@@ -115,16 +139,21 @@ class RoutedExperts(FeedForward):
         rows = [tensors["router"]] + ([tensors["shared.score"]] if self.shared_gate else [])
         # the router (and the shared expert's score) are one product, its result 32-bit
         self.router = as_product_weight(torch.cat(rows, dim=0).contiguous())
-        self.gate_w = stack_experts(tensors[f"e{e}.gate"] for e in range(E))
+        self.gate_w = stack_experts(tensors[f"e{e}.gate"] for e in range(E)) if self.gated else None
         self.up_w = stack_experts(tensors[f"e{e}.up"] for e in range(E))
         self.down_w = stack_experts(tensors[f"e{e}.down"] for e in range(E))
+        self.correction_w = tensors["correction"].contiguous() if self.correction else None
         if self.shared is not None:
             self.shared.load({n: tensors["shared." + n] for n in self.shared.param_specs()})
 
     def forward(self, x: torch.Tensor, ctx=None) -> torch.Tensor:
         E = self.num_experts
         logits = ops.gemm(x, self.router, out_dtype=torch.float32)
-        experts, weights = ops.route(logits[:, :E], self.top, self.router_scale)
+        if self.router_kind == "sigmoid":
+            experts, weights = ops.route_choice(logits[:, :E], self.top, self.router_scale, correction=self.correction_w,
+                                                groups=self.num_groups, keep=self.keep_groups)
+        else:
+            experts, weights = ops.route(logits[:, :E], self.top, self.router_scale)
         shared = self.shared.forward(x, ctx) if self.shared is not None else None
         return ops.routed_experts(x, experts, weights, self.gate_w, self.up_w, self.down_w, self.activation_code,
                                   shared=shared, shared_gate=logits[:, E:E + 1] if self.shared_gate else None)

@@ -35,7 +35,8 @@ def cpu_ops(monkeypatch):
                  "residual_add_norm", "gated_heads", "activation_", "qk_norm_rope_cache_write", "short_conv_silu",
                  "delta_prepare", "delta_inputs", "delta_rule", "embed_sum", "token_gate_", "bias_add_", "weighted_sum",
                  "exp_gates", "linear_state", "normalized_readout", "route", "routed_experts", "residual_add_next_norm",
-                 "paged_attention_maps", "attention_maps_units_takes", "norm_rope_cache_write", "short_conv", "head_product", "rglru_scan"):
+                 "paged_attention_maps", "attention_maps_units_takes", "norm_rope_cache_write", "short_conv", "head_product", "rglru_scan",
+                 "attention_inputs", "route_choice"):
         monkeypatch.setattr(ops, name, getattr(torch_ops, name))
     return torch_ops
 

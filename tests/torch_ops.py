@@ -209,7 +209,7 @@ def decode_attention_takes(q, k_pages, num_heads, max_q_len):
 
 
 def paged_attention_sink(q, k_pages, v_pages, block_table, token_seq, positions, num_heads, *, scale=1.0, sinks=None,
-                         window=None, soft_cap=None, out=None):
+                         window=None, soft_cap=None, out=None, slopes=None):
     T = q.shape[0]
     _, Kh, P, dk = k_pages.shape
     dv = v_pages.shape[2]
@@ -229,6 +229,8 @@ def paged_attention_sink(q, k_pages, v_pages, block_table, token_seq, positions,
         s = torch.einsum("kgd,nkd->kgn", qt, k) * scale
         if soft_cap:
             s = soft_cap * torch.tanh(s / soft_cap)
+        if slopes is not None:
+            s = s - _f(slopes).reshape(Kh, G, 1) * (pos - keys).to(s.dtype)[None, None, :]
         if sinks is not None:
             s = torch.cat([s, _f(sinks).reshape(Kh, G, 1)], dim=-1)
         p = torch.softmax(s, -1)[..., :len(keys)]
@@ -259,12 +261,12 @@ def residual_add_norm(y, residual, *, weight=None, eps=0.0, plus_one=False, mult
 GATE_SIGMOID, GATE_SILU = 0, 1
 
 
-def gated_heads(x, gate, num_heads, size, *, kind, weight=None, eps=0.0, out_dtype=None, out=None):
+def gated_heads(x, gate, num_heads, size, *, kind, weight=None, eps=0.0, out_dtype=None, out=None, per_head=False):
     T = x.shape[0]
     v = _f(x).reshape(T, num_heads, size)
     if weight is not None:
         v = v / torch.sqrt((v * v).mean(-1, keepdim=True) + eps) * _f(weight)
-    g = _f(gate).reshape(T, num_heads, size)
+    g = _f(gate).reshape(T, num_heads, 1 if per_head else size)
     g = torch.sigmoid(g) if kind == GATE_SIGMOID else g * torch.sigmoid(g)
     r = (v * g).reshape(T, num_heads * size).to(out_dtype or (out.dtype if out is not None else x.dtype))
     if out is not None:
@@ -582,6 +584,21 @@ def route(logits, top, scale):
     return best.indices.to(torch.int32).contiguous(), (best.values * scale).to(torch.float32).contiguous()
 
 
+def route_choice(logits, top, scale, *, correction=None, groups=1, keep=1):
+    s = torch.sigmoid(_f(logits))
+    T, E = s.shape
+    c = s + _f(correction) if correction is not None else s.clone()
+    if groups > 1:
+        per = E // groups
+        by_group = c.reshape(T, groups, per)
+        score = torch.topk(by_group, min(2, per), dim=-1).values.sum(-1)
+        stay = torch.zeros(T, groups, dtype=torch.bool, device=s.device)
+        stay.scatter_(1, torch.topk(score, keep, dim=-1).indices, True)
+        c = torch.where(stay[:, :, None].expand(T, groups, per).reshape(T, E), c, torch.full_like(c, float("-inf")))
+    chosen = torch.topk(c, top, dim=-1).indices
+    return chosen.to(torch.int32).contiguous(), (torch.gather(s, 1, chosen) * scale).to(torch.float32).contiguous()
+
+
 def routed_experts(x, experts, weights, gate_w, up_w, down_w, activation, *, shared=None, shared_gate=None,
                    out_dtype=None):
     from simply_amd.kernels.packing import TiledWeight, unpack_tiles
@@ -597,8 +614,11 @@ def routed_experts(x, experts, weights, gate_w, up_w, down_w, activation, *, sha
     for t in range(T):
         for k in range(experts.shape[1]):
             e = int(experts[t, k])
-            h = _activation(activation, (xf[t] @ matrix(gate_w, e).T).to(x.dtype).to(xf.dtype)) \
-                * (xf[t] @ matrix(up_w, e).T).to(x.dtype).to(xf.dtype)
+            if gate_w is None:   # experts without a gate
+                h = _activation(activation, (xf[t] @ matrix(up_w, e).T).to(x.dtype).to(xf.dtype))
+            else:
+                h = _activation(activation, (xf[t] @ matrix(gate_w, e).T).to(x.dtype).to(xf.dtype)) \
+                    * (xf[t] @ matrix(up_w, e).T).to(x.dtype).to(xf.dtype)
             out[t] += _f(weights[t, k]) * (h.to(x.dtype).to(xf.dtype) @ matrix(down_w, e).T)
     if shared is not None:
         s = _f(shared)
@@ -753,3 +773,60 @@ def rglru_scan(u, gates, block, r_bias, i_bias, lam, y, y_bias, state, seq_meta,
             out[t] = (S * gy[t]).to(out.dtype)
         state[slot, :C] = S.to(torch.float32)
     return out
+
+
+# --------------------------------------------------------------------------- what a windowed attention reads
+
+
+def attention_inputs(proj, seq_meta, num_seqs, max_q_len, num_heads, num_kv_heads, key_dim, value_dim, *,
+                     values_are_keys=False, taps=None, tails=None, norm=None, q_weight=None, k_weight=None, eps=0.0,
+                     inv_freq=None, rot_dims=0, temp_coef=0.0, temp_every=0, slot_mapping=None, k_pages=None,
+                     v_pages=None):
+    H, K, dk, dv = num_heads, num_kv_heads, key_dim, value_dim
+    own = k_pages is not None
+    C = (H + K) * dk + (0 if values_are_keys else K * dv) if own else H * dk
+    T = proj.shape[0]
+    x = _f(proj[:, :C]).clone()
+    if taps is not None:
+        n, w = taps.shape[1], _f(taps)
+        for slot, first, count, _ in seq_meta[:num_seqs].tolist():
+            new = x[first:first + count].clone()
+            old = _f(tails[slot, :(n - 1) * C]).reshape(n - 1, C) if n > 1 else new[:0]
+            xs = torch.cat([old, new], dim=0)
+            x[first:first + count] = sum(xs[j:j + count] * w[:, j][None, :] for j in range(n))
+            if n > 1:
+                tails[slot, :(n - 1) * C] = xs[count:].reshape(-1).to(torch.float32)
+    pos = torch.empty(T, dtype=torch.long, device=proj.device)
+    for slot, first, count, start in seq_meta[:num_seqs].tolist():
+        pos[first:first + count] = torch.arange(start, start + count, device=proj.device)
+
+    def prepared(rows, heads, weight):
+        v = rows.reshape(T, heads, dk)
+        if norm == "head":
+            v = v / torch.sqrt((v * v).mean(-1, keepdim=True) + eps) * _f(weight)
+        elif norm == "row":
+            flat = v.reshape(T, heads * dk)
+            v = (flat / torch.sqrt((flat * flat).mean(-1, keepdim=True) + eps) * _f(weight)).reshape(T, heads, dk)
+        if rot_dims:
+            half = rot_dims // 2
+            a = pos.to(torch.float32)[:, None] * inv_freq.to(torch.float32)[None, :]
+            cos, sin = torch.cos(a).to(v.dtype)[:, None, :], torch.sin(a).to(v.dtype)[:, None, :]
+            u, w_ = v[..., :half], v[..., half:rot_dims]
+            v = torch.cat([u * cos - w_ * sin, w_ * cos + u * sin, v[..., rot_dims:]], dim=-1)
+        return v
+
+    q = prepared(x[:, :H * dk], H, q_weight)
+    if temp_every:
+        q = q * (1.0 + temp_coef * torch.log(torch.floor((pos + 1) / temp_every) + 1.0)).to(q.dtype)[:, None, None]
+    if own:
+        k_raw = x[:, H * dk:(H + K) * dk]
+        k = prepared(k_raw, K, k_weight)
+        v = k_raw.reshape(T, K, dk) if values_are_keys else x[:, (H + K) * dk:C].reshape(T, K, dv)
+        P = k_pages.shape[2]
+        rows = stored_keys_as_rows(k_pages)
+        keep = slot_mapping[:T] >= 0
+        page, off = (slot_mapping[:T] // P)[keep], (slot_mapping[:T] % P)[keep]
+        rows[page, :, off] = k[keep].to(k_pages.dtype)
+        k_pages.copy_(rows_as_stored_keys(rows))
+        v_pages[page, :, :, off] = v[keep].to(v_pages.dtype)
+    return q.reshape(T, H * dk).to(proj.dtype)
