@@ -246,7 +246,7 @@ int paged_attention_decode(const void* q, int64_t q_stride, const void* k_pages,
                            const int* block_table, int table_stride, const int* seq_meta, int seq_begin, int seq_count,
                            void* out, int64_t out_stride, int H, int Kh, int hd, int page_size, int window,
                            float soft_cap, int max_kv_len, int max_q_len, int num_splits, void* workspace, size_t workspace_bytes,
-                           hipStream_t stream, const float* sinks = nullptr);
+                           hipStream_t stream, const float* sinks = nullptr, const float* slopes = nullptr);
 int paged_attention_prefill_group();  // units that one workgroup takes
 bool paged_attention_prefill_takes(int H, int Kh, int hd, int page_size, int max_q_len, int64_t q_stride, const void* q,
                                    int64_t out_stride, const void* out);
@@ -254,7 +254,7 @@ int paged_attention_prefill(const void* q, int64_t q_stride, const void* k_pages
                             const int* block_table, int table_stride, const int* units, int unit_begin, int unit_count,
                             void* out, int64_t out_stride, int H, int Kh, int hd, int page_size, int window,
                             float soft_cap, int max_kv_len, int max_q_len, int num_splits, void* workspace, size_t workspace_bytes,
-                            hipStream_t stream, const float* sinks = nullptr);
+                            hipStream_t stream, const float* sinks = nullptr, const float* slopes = nullptr);
 bool gemm_wide_takes(int M, int N, int K, int64_t lda, int64_t ldc, const void* A, const void* W, const void* W2,
                      const void* C, int c_dtype, int epi, int packed);
 int gemm_wide(const void* A, int64_t lda, const void* W, void* C, int64_t ldc, int M, int N, int K, int epi, int act,
@@ -413,17 +413,20 @@ int sa_delta_rule(const float* qkv, int C, int G, int dk, int dv, const float* g
                   int64_t state_stride, const int* seq_meta, int num_seqs, float* out, hipStream_t stream);
 
 // sa_paged_attention_decode and sa_paged_attention_prefill for softmax sums that hold one more term per query head,
-// exp(sinks[h]) (float32 [H]; null: none), without a value.
+// exp(sinks[h]) (float32 [H]; null: none), without a value, and with slopes (float32 [H]; null: none): slopes[h] times
+// the distance between query and key is taken off the score.
 int sa_paged_attention_decode_sink(const void* q, int64_t q_stride, const void* k_pages, const void* v_pages,
                                    const int* block_table, int table_stride, const int* seq_meta, int seq_begin,
                                    int seq_count, void* out, int64_t out_stride, int H, int Kh, int hd, int page_size,
                                    int window, float soft_cap, int max_kv_len, int max_q_len, int num_splits,
-                                   void* workspace, int64_t workspace_bytes, const float* sinks, hipStream_t stream);
+                                   void* workspace, int64_t workspace_bytes, const float* sinks, const float* slopes,
+                                    hipStream_t stream);
 int sa_paged_attention_prefill_sink(const void* q, int64_t q_stride, const void* k_pages, const void* v_pages,
                                     const int* block_table, int table_stride, const int* seq_meta, int unit_begin,
                                     int unit_count, void* out, int64_t out_stride, int H, int Kh, int hd, int page_size,
                                     int window, float soft_cap, int max_kv_len, int max_q_len, int num_splits,
-                                    void* workspace, int64_t workspace_bytes, const float* sinks, hipStream_t stream);
+                                    void* workspace, int64_t workspace_bytes, const float* sinks, const float* slopes,
+                                    hipStream_t stream);
 // ---- token tables
 // out[t, :] = table[token] + pair[(previous * mul_prev + token * mul_cur) mod buckets] + pos[position]; a request's
 // first token takes the pair table's row `buckets`; the token before a step's first one is last[slot], which is then
@@ -468,12 +471,12 @@ int sa_normalized_readout(const float* x, const float* floor, int64_t floor_stri
 // 0: none; 1: queries and keys head by head with weights [dk]; 2: over the whole row with weights [H * dk] and
 // [K * dk].  Then the first rot_dims entries of every head turn in pairs (i, i + rot_dims / 2) by position *
 // inv_freq[i], and queries are multiplied by 1 + temp_coef * ln(floor((position + 1) / temp_every) + 1) (temp_every 0:
-// not).  Queries go to q_out [T, H * dk], keys and values into their pages.
+// not) and by q_mult.  Queries go to q_out [T, H * dk], keys and values into their pages.
 int sa_attention_inputs(const void* proj, int dtype, int64_t row_stride, int H, int K, int dk, int dv, int k_at, int v_at,
                         int values_are_keys, const void* taps, int taps_dtype, int num_taps, float* tails,
                         int64_t tail_stride, int norm, const void* q_w, const void* k_w, int w_dtype, float eps,
-                        const float* inv_freq, int rot_dims, float temp_coef, int temp_every, const int* seq_meta,
-                        int num_seqs, int max_q_len, const int64_t* slot_mapping, void* q_out, int64_t q_stride,
+                        const float* inv_freq, int rot_dims, float temp_coef, int temp_every, float q_mult,
+                        const int* seq_meta, int num_seqs, int max_q_len, const int64_t* slot_mapping, void* q_out, int64_t q_stride,
                         void* k_pages, void* v_pages, int page_size, hipStream_t stream);
 
 // ---- routed experts (routed.hip)

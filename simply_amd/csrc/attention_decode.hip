@@ -43,8 +43,9 @@ __global__ __launch_bounds__(256) void paged_attention_decode_kernel(
     const bf16* __restrict__ q, int64_t q_stride, const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
     const int* __restrict__ block_table, int table_stride, const SeqMeta* __restrict__ seq_meta, int seq_begin,
     bf16* __restrict__ out, int64_t out_stride, int Kh, int G, int page_size, int window, float soft_cap,
-    float* __restrict__ workspace, const float* __restrict__ sinks) {
+    float* __restrict__ workspace, const float* __restrict__ sinks, const float* __restrict__ slopes) {
   // sinks (or null): one logit per query head that joins the softmax's sum and has no value
+  // slopes (or null): per query head, what a score loses for every position between the query and the key
   constexpr int HD = NDC * 32;
   constexpr int NDB = HD / 16;  // output blocks of 16 dimensions
   __shared__ __align__(16) float o_s[2][16][HD + 4];   // a wave's output [row][d], while two waves are merged (rows of 16-byte pieces)
@@ -66,6 +67,7 @@ __global__ __launch_bounds__(256) void paged_attention_decode_kernel(
   const int hi = sm.pos0 + sm.q_len;  // keys [lo, hi) are visible to some row
   const int lo = (window > 0 && sm.pos0 - window + 1 > 0) ? sm.pos0 - window + 1 : 0;
   const int lo_r = (window > 0 && pos_r - window + 1 > 0) ? pos_r - window + 1 : 0;
+  const float slope_r = slopes != nullptr ? slopes[kh * G + g] : 0.f;
 
   // tiles of 32 keys aligned to absolute positions; this workgroup's share, then this wave's
   const int tile0 = lo / kTile, tile1 = (hi + kTile - 1) / kTile;
@@ -192,6 +194,7 @@ __global__ __launch_bounds__(256) void paged_attention_decode_kernel(
         const int key = key0 + t * 16 + grp * 4 + v;
         float x = s[t][v];
         if (soft_cap > 0.f) x = soft_cap * fast_tanh(x / soft_cap);
+        if (slopes != nullptr) x -= slope_r * static_cast<float>(pos_r - key);
         const bool vis = sub_ok[t] && row_ok && key <= pos_r && key >= lo_r;
         x = vis ? x : -INFINITY;
         p[t][v] = x;
@@ -447,7 +450,7 @@ int paged_attention_decode(const void* q, int64_t q_stride, const void* k_pages,
                            const int* block_table, int table_stride, const int* seq_meta, int seq_begin, int seq_count,
                            void* out, int64_t out_stride, int H, int Kh, int hd, int page_size, int window,
                            float soft_cap, int max_kv_len, int max_q_len, int num_splits, void* workspace, size_t workspace_bytes,
-                           hipStream_t stream, const float* sinks) {
+                           hipStream_t stream, const float* sinks, const float* slopes) {
   if (seq_count == 0) return 0;
   const int G = H / Kh;
   const int units = seq_count * Kh;
@@ -466,7 +469,7 @@ int paged_attention_decode(const void* q, int64_t q_stride, const void* k_pages,
 #define SA_LAUNCH(NDC)                                                                                              \
   paged_attention_decode_kernel<NDC><<<grid, 256, 0, stream>>>(qp, q_stride, kp, vp, block_table, table_stride, sm, \
                                                                seq_begin, op, out_stride, Kh, G, page_size, window,  \
-                                                               soft_cap, ws, sinks)
+                                                               soft_cap, ws, sinks, slopes)
   if (hd == 64) SA_LAUNCH(2);
   else if (hd == 128) SA_LAUNCH(4);
   else if (hd == 256) SA_LAUNCH(8);

@@ -9,7 +9,8 @@
 //                 heads; or over the whole row (all heads at once) with a weight per entry.
 //   rotation      the first rot_dims entries of every head turn, entry i with entry i + rot_dims / 2, by the angle
 //                 position * inv_freq[i]; after the norm.
-//   temperature   queries at position p times 1 + coef * ln(floor((p + 1) / every) + 1)  (every == 0: none).
+//   temperature   queries at position p times 1 + coef * ln(floor((p + 1) / every) + 1)  (every == 0: none), and times
+//                 q_mult (the scores' factor, for an attention kernel that has none of its own).
 //   values        their own columns of the projection (convolved, otherwise as they are), or the keys' columns as they
 //                 stand before norm and rotation.
 //
@@ -35,6 +36,7 @@ struct AttentionInputs {
   int rot_dims;
   int temp_every;
   float temp_coef, eps;
+  float q_mult;             // a factor on the queries (the scores' factor, for an attention kernel that has none)
   int page_size;
 };
 
@@ -109,8 +111,8 @@ __global__ __launch_bounds__(kInputThreads) void attention_inputs_kernel(
     r_all = 1.f / sqrtf(block_sum(ss, red_s) / static_cast<float>(len) + p.eps);
   }
   const float temp = (sec == 0 && p.temp_every > 0)
-                         ? 1.f + p.temp_coef * logf(static_cast<float>((pos + 1) / p.temp_every) + 1.f)
-                         : 1.f;
+                         ? (1.f + p.temp_coef * logf(static_cast<float>((pos + 1) / p.temp_every) + 1.f)) * p.q_mult
+                         : p.q_mult;
   const int half = p.rot_dims / 2;
   const bool tiled = keys_tiled(p.page_size, p.dk);
   T* kdst = sec == 1 ? k_pages + (page * p.K) * p.page_size * p.dk : nullptr;
@@ -164,7 +166,8 @@ extern "C" int sa_attention_inputs(const void* proj, int dtype, int64_t row_stri
                                    int k_at, int v_at, int values_are_keys, const void* taps, int taps_dtype,
                                    int num_taps, float* tails, int64_t tail_stride, int norm, const void* q_w,
                                    const void* k_w, int w_dtype, float eps, const float* inv_freq, int rot_dims,
-                                   float temp_coef, int temp_every, const int* seq_meta, int num_seqs, int max_q_len,
+                                   float temp_coef, int temp_every, float q_mult, const int* seq_meta, int num_seqs,
+                                   int max_q_len,
                                    const int64_t* slot_mapping, void* q_out, int64_t q_stride, void* k_pages,
                                    void* v_pages, int page_size, hipStream_t stream) {
   if (num_seqs == 0 || max_q_len == 0) return 0;
@@ -203,7 +206,7 @@ extern "C" int sa_attention_inputs(const void* proj, int dtype, int64_t row_stri
   AttentionInputs p;
   p.H = H, p.K = K, p.dk = dk, p.dv = dv, p.k_at = k_at, p.v_at = v_at, p.values_are_keys = values_are_keys;
   p.taps = num_taps, p.conv_channels = C, p.norm = norm, p.rot_dims = rot_dims, p.temp_every = temp_every;
-  p.temp_coef = temp_coef, p.eps = eps, p.page_size = page_size;
+  p.temp_coef = temp_coef, p.eps = eps, p.page_size = page_size, p.q_mult = q_mult;
   const dim3 grid(max_q_len, num_seqs, own ? (values_are_keys ? 2 : 3) : 1);
   const dim3 tail_grid((C + kWave - 1) / kWave, num_seqs);
   if (dtype == kF32) {

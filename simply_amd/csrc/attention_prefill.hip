@@ -58,8 +58,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(R == 1 ? 2 
     const bf16* __restrict__ q, int64_t q_stride, const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
     const int* __restrict__ block_table, int table_stride, const SeqMeta* __restrict__ units, int unit_begin,
     bf16* __restrict__ out, int64_t out_stride, int Kh, int G, int page_size, int window, float soft_cap,
-    float* __restrict__ workspace, int chunk_tiles, const float* __restrict__ sinks) {
+    float* __restrict__ workspace, int chunk_tiles, const float* __restrict__ sinks,
+    const float* __restrict__ slopes) {
   // sinks (or null): one logit per query head that joins the softmax's sum and has no value
+  // slopes (or null): per query head, what a score loses for every position between the query and the key
   constexpr int HD = NDC * 32;
   constexpr int NDB = HD / 16;            // output blocks of 16 dimensions
   constexpr int CPW = NDC / 2;            // KiB chunks of keys (and of values) per wave and tile
@@ -126,6 +128,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(R == 1 ? 2 
   }
 
   // scores in base-2 units: y = log2(e) * cap * tanh(s / cap) = c2 - 2 * c2 / (2^(s * c1) + 1), or log2(e) * s
+  const float slope2 = slopes != nullptr ? slopes[kh * G + g] * kLog2e : 0.f;
   const float c1 = CAP ? 2.f * kLog2e / soft_cap : kLog2e;
   const float c2 = soft_cap * kLog2e;
 
@@ -283,6 +286,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(R == 1 ? 2 
           if (CAP) x = c2 - 2.f * c2 * __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(x) + 1.f);
           y[t][v] = x;
         }
+      if (slopes != nullptr) {  // uniform over the launch: the distance bias, in the base-2 scale of the scores
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int v = 0; v < 4; ++v)
+            y[t][v] -= slope2 * static_cast<float>(pos_r[j] - (key0 + grp * 8 + t * 4 + v));
+      }
       if (!whole) {  // uniform over the wave
 #pragma unroll
         for (int t = 0; t < 2; ++t)
@@ -420,7 +430,7 @@ int paged_attention_prefill(const void* q, int64_t q_stride, const void* k_pages
                             const int* block_table, int table_stride, const int* units, int unit_begin, int unit_count,
                             void* out, int64_t out_stride, int H, int Kh, int hd, int page_size, int window,
                             float soft_cap, int max_kv_len, int max_q_len, int num_splits, void* workspace, size_t workspace_bytes,
-                            hipStream_t stream, const float* sinks) {
+                            hipStream_t stream, const float* sinks, const float* slopes) {
   constexpr int R = kPrefillRowTiles;
   constexpr int kGroup = prefill::kWaves * R;
   if (unit_count == 0) return 0;
@@ -466,11 +476,11 @@ int paged_attention_prefill(const void* q, int64_t q_stride, const void* k_pages
     if (soft_cap > 0.f)                                                                                             \
       prefill::paged_attention_prefill_kernel<NDC, R, true><<<grid, 256, 0, stream>>>(                              \
           qp, q_stride, kp, vp, block_table, table_stride, um, unit_begin, op, out_stride, Kh, G, page_size, window, \
-          soft_cap, ws, chunk, sinks);                                                                              \
+          soft_cap, ws, chunk, sinks, slopes);                                                                        \
     else                                                                                                            \
       prefill::paged_attention_prefill_kernel<NDC, R, false><<<grid, 256, 0, stream>>>(                             \
           qp, q_stride, kp, vp, block_table, table_stride, um, unit_begin, op, out_stride, Kh, G, page_size, window, \
-          soft_cap, ws, chunk, sinks);                                                                              \
+          soft_cap, ws, chunk, sinks, slopes);                                                                        \
   } while (0)
   if (hd == 64) SA_LAUNCH(2);
   else if (hd == 128) SA_LAUNCH(4);

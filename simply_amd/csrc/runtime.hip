@@ -223,7 +223,7 @@ extern "C" int sa_paged_attention_decode_sink(const void* q, int64_t q_stride, c
                                               int64_t out_stride, int H, int Kh, int hd, int page_size, int window,
                                               float soft_cap, int max_kv_len, int max_q_len, int num_splits,
                                               void* workspace, int64_t workspace_bytes, const float* sinks,
-                                              hipStream_t stream);
+                                              const float* slopes, hipStream_t stream);
 extern "C" int sa_paged_attention_decode(const void* q, int64_t q_stride, const void* k_pages, const void* v_pages,
                                          const int* block_table, int table_stride, const int* seq_meta, int seq_begin,
                                          int seq_count, void* out, int64_t out_stride, int H, int Kh, int hd,
@@ -232,7 +232,7 @@ extern "C" int sa_paged_attention_decode(const void* q, int64_t q_stride, const 
                                          hipStream_t stream) {
   return sa_paged_attention_decode_sink(q, q_stride, k_pages, v_pages, block_table, table_stride, seq_meta, seq_begin,
                                         seq_count, out, out_stride, H, Kh, hd, page_size, window, soft_cap, max_kv_len,
-                                        max_q_len, num_splits, workspace, workspace_bytes, nullptr, stream);
+                                        max_q_len, num_splits, workspace, workspace_bytes, nullptr, nullptr, stream);
 }
 
 extern "C" int sa_paged_attention_decode_sink(const void* q, int64_t q_stride, const void* k_pages,
@@ -241,7 +241,7 @@ extern "C" int sa_paged_attention_decode_sink(const void* q, int64_t q_stride, c
                                               int64_t out_stride, int H, int Kh, int hd, int page_size, int window,
                                               float soft_cap, int max_kv_len, int max_q_len, int num_splits,
                                               void* workspace, int64_t workspace_bytes, const float* sinks,
-                                              hipStream_t stream) {
+                                              const float* slopes, hipStream_t stream) {
   if (seq_count == 0) return 0;
   SA_REQUIRE(seq_count > 0 && seq_begin >= 0 && H > 0 && Kh > 0 && H % Kh == 0, "paged_attention_decode: bad counts");
   SA_REQUIRE(window >= 0 && table_stride > 0 && max_kv_len > 0, "paged_attention_decode: bad window, table or length");
@@ -251,7 +251,8 @@ extern "C" int sa_paged_attention_decode_sink(const void* q, int64_t q_stride, c
   SA_REQUIRE(out_stride >= static_cast<int64_t>(H) * hd, "paged_attention_decode: output rows are too short");
   return paged_attention_decode(q, q_stride, k_pages, v_pages, block_table, table_stride, seq_meta, seq_begin, seq_count,
                                 out, out_stride, H, Kh, hd, page_size, window, soft_cap, max_kv_len, max_q_len, num_splits,
-                                workspace, static_cast<size_t>(workspace_bytes < 0 ? 0 : workspace_bytes), stream, sinks);
+                                workspace, static_cast<size_t>(workspace_bytes < 0 ? 0 : workspace_bytes), stream, sinks,
+                                slopes);
 }
 
 extern "C" int sa_paged_attention_decode_takes(int H, int Kh, int hd, int page_size, int max_q_len, int64_t q_stride,
@@ -267,7 +268,7 @@ extern "C" int sa_paged_attention_prefill_sink(const void* q, int64_t q_stride, 
                                                int64_t out_stride, int H, int Kh, int hd, int page_size, int window,
                                                float soft_cap, int max_kv_len, int max_q_len, int num_splits,
                                                void* workspace, int64_t workspace_bytes, const float* sinks,
-                                               hipStream_t stream);
+                                               const float* slopes, hipStream_t stream);
 extern "C" int sa_paged_attention_prefill(const void* q, int64_t q_stride, const void* k_pages, const void* v_pages,
                                           const int* block_table, int table_stride, const int* seq_meta, int unit_begin,
                                           int unit_count, void* out, int64_t out_stride, int H, int Kh, int hd,
@@ -276,7 +277,7 @@ extern "C" int sa_paged_attention_prefill(const void* q, int64_t q_stride, const
                                           hipStream_t stream) {
   return sa_paged_attention_prefill_sink(q, q_stride, k_pages, v_pages, block_table, table_stride, seq_meta, unit_begin,
                                          unit_count, out, out_stride, H, Kh, hd, page_size, window, soft_cap, max_kv_len,
-                                         max_q_len, num_splits, workspace, workspace_bytes, nullptr, stream);
+                                         max_q_len, num_splits, workspace, workspace_bytes, nullptr, nullptr, stream);
 }
 
 extern "C" int sa_paged_attention_prefill_sink(const void* q, int64_t q_stride, const void* k_pages,
@@ -285,7 +286,7 @@ extern "C" int sa_paged_attention_prefill_sink(const void* q, int64_t q_stride, 
                                                int64_t out_stride, int H, int Kh, int hd, int page_size, int window,
                                                float soft_cap, int max_kv_len, int max_q_len, int num_splits,
                                                void* workspace, int64_t workspace_bytes, const float* sinks,
-                                               hipStream_t stream) {
+                                               const float* slopes, hipStream_t stream) {
   if (unit_count == 0) return 0;
   SA_REQUIRE(unit_count > 0 && unit_count % paged_attention_prefill_group() == 0 && unit_begin >= 0 && H > 0 && Kh > 0 &&
                  H % Kh == 0,
@@ -299,5 +300,5 @@ extern "C" int sa_paged_attention_prefill_sink(const void* q, int64_t q_stride, 
   return paged_attention_prefill(q, q_stride, k_pages, v_pages, block_table, table_stride, seq_meta, unit_begin,
                                  unit_count, out, out_stride, H, Kh, hd, page_size, window, soft_cap, max_kv_len,
                                  max_q_len, num_splits, workspace, static_cast<size_t>(workspace_bytes < 0 ? 0 : workspace_bytes),
-                                 stream, sinks);
+                                 stream, sinks, slopes);
 }

@@ -625,8 +625,8 @@ def decode_attention_takes(q: torch.Tensor, k_pages: torch.Tensor, num_heads: in
 
 
 def _attention_units(entry: str, q, k_pages, v_pages, block_table, seq_meta, begin, count, num_heads, window, soft_cap,
-                     max_kv_len, max_q_len, out, num_splits, sinks=None):
-    _dev(q, k_pages, v_pages, block_table, seq_meta, out, sinks)
+                     max_kv_len, max_q_len, out, num_splits, sinks=None, slopes=None):
+    _dev(q, k_pages, v_pages, block_table, seq_meta, out, sinks, slopes)
     name = entry[3:]
     if q.dtype != torch.bfloat16:
         raise KernelError(f"{name}: bfloat16 only")
@@ -642,14 +642,17 @@ def _attention_units(entry: str, q, k_pages, v_pages, block_table, seq_meta, beg
         raise KernelError(f"{name}: bad output")
     out_stride = _rows(out, f"{name}: out")
     ws = _workspace(q.device)
-    if sinks is not None:
-        # one more term exp(sinks[h]) in every softmax sum of query head h, without a value
-        if sinks.dtype != torch.float32 or sinks.numel() != num_heads or not sinks.is_contiguous():
-            raise KernelError(f"{name}: sinks must be contiguous float32, one per query head")
+    if sinks is not None or slopes is not None:
+        # one more term exp(sinks[h]) in every softmax sum of query head h, without a value; slopes[h] times the
+        # distance between query and key taken off the scores
+        for per_head in (sinks, slopes):
+            if per_head is not None and (per_head.dtype != torch.float32 or per_head.numel() != num_heads
+                                         or not per_head.is_contiguous()):
+                raise KernelError(f"{name}: sinks and slopes must be contiguous float32, one per query head")
         _lib.call(entry + "_sink", _ptr(q), q_stride, _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
                   block_table.stride(0), _ptr(seq_meta), begin, count, _ptr(out), out_stride, num_heads, Kh, hd,
                   page_size, int(window or 0), float(soft_cap or 0.0), int(max_kv_len), int(max_q_len), int(num_splits),
-                  _ptr(ws), ws.numel(), _ptr(sinks), _stream())
+                  _ptr(ws), ws.numel(), _ptr(sinks), _ptr(slopes), _stream())
         return out
     _lib.call(entry, _ptr(q), q_stride, _ptr(k_pages), _ptr(v_pages), _ptr(block_table),
               block_table.stride(0), _ptr(seq_meta), begin, count, _ptr(out), out_stride, num_heads, Kh, hd,
@@ -661,12 +664,14 @@ def _attention_units(entry: str, q, k_pages, v_pages, block_table, seq_meta, beg
 def paged_attention_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,
                            seq_meta: torch.Tensor, seq_begin: int, seq_count: int, num_heads: int, *,
                            window: int | None, soft_cap: float | None, max_kv_len: int, max_q_len: int,
-                           out: torch.Tensor, num_splits: int = 0, sinks: torch.Tensor | None = None) -> torch.Tensor:
+                           out: torch.Tensor, num_splits: int = 0, sinks: torch.Tensor | None = None,
+                           slopes: torch.Tensor | None = None) -> torch.Tensor:
     """Attention of requests seq_begin .. seq_begin + seq_count - 1 of seq_meta, each with few tokens
     ((heads per key head) * tokens <= 16).  q and out are the whole step's rows.  sinks: float32 [H], one more term
-    exp(sinks[h]) in every softmax sum, without a value."""
+    exp(sinks[h]) in every softmax sum, without a value.  slopes: float32 [H], slopes[h] times the distance between
+    query and key is taken off the scores."""
     return _attention_units("sa_paged_attention_decode", q, k_pages, v_pages, block_table, seq_meta, seq_begin,
-                            seq_count, num_heads, window, soft_cap, max_kv_len, max_q_len, out, num_splits, sinks)
+                            seq_count, num_heads, window, soft_cap, max_kv_len, max_q_len, out, num_splits, sinks, slopes)
 
 
 def prefill_units_per_group() -> int:
@@ -677,7 +682,8 @@ def prefill_units_per_group() -> int:
 def paged_attention_prefill(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,
                             units: torch.Tensor, unit_begin: int, unit_count: int, num_heads: int, *,
                             window: int | None, soft_cap: float | None, max_kv_len: int, max_q_len: int,
-                            out: torch.Tensor, num_splits: int = 0, sinks: torch.Tensor | None = None) -> torch.Tensor:
+                            out: torch.Tensor, num_splits: int = 0, sinks: torch.Tensor | None = None,
+                            slopes: torch.Tensor | None = None) -> torch.Tensor:
     """Attention of portions of prompts cut into units of few tokens ((heads per key head) * tokens <= 16), rows
     unit_begin .. unit_begin + unit_count - 1 of `units` in the layout of seq_meta.  One workgroup takes a group of
     consecutive units, which must belong to one request (units without tokens fill up the last group), and
@@ -685,7 +691,7 @@ def paged_attention_prefill(q: torch.Tensor, k_pages: torch.Tensor, v_pages: tor
     if unit_count % prefill_units_per_group():
         raise KernelError(f"paged_attention_prefill: units come in groups of {prefill_units_per_group()}")
     return _attention_units("sa_paged_attention_prefill", q, k_pages, v_pages, block_table, units, unit_begin,
-                            unit_count, num_heads, window, soft_cap, max_kv_len, max_q_len, out, num_splits, sinks)
+                            unit_count, num_heads, window, soft_cap, max_kv_len, max_q_len, out, num_splits, sinks, slopes)
 
 
 def paged_attention_sink(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,
@@ -990,7 +996,7 @@ def attention_inputs(proj: torch.Tensor, seq_meta: torch.Tensor, num_seqs: int, 
                      taps: torch.Tensor | None = None, tails: torch.Tensor | None = None, norm: str | None = None,
                      q_weight: torch.Tensor | None = None, k_weight: torch.Tensor | None = None, eps: float = 0.0,
                      inv_freq: torch.Tensor | None = None, rot_dims: int = 0, temp_coef: float = 0.0, temp_every: int = 0,
-                     slot_mapping: torch.Tensor | None = None, k_pages: torch.Tensor | None = None,
+                     q_mult: float = 1.0, slot_mapping: torch.Tensor | None = None, k_pages: torch.Tensor | None = None,
                      v_pages: torch.Tensor | None = None) -> torch.Tensor:
     """From fused projection rows [H * dk queries | K * dk keys | K * dv values | ...] of a ragged step (seq_meta) to
     what an attention kernel reads.  taps [channels, n] with tails float32 [slots, (n - 1) * channels]: every channel
@@ -998,7 +1004,7 @@ def attention_inputs(proj: torch.Tensor, seq_meta: torch.Tensor, num_seqs: int, 
     are brought up to date).  norm 'head': queries and keys divided by each head's root mean square, times q_weight /
     k_weight [dk]; 'row': by the whole row's, times weights [H * dk] / [K * dk].  Then the first rot_dims entries of
     every head turn in pairs (i, i + rot_dims / 2) by position * inv_freq[i]; queries are multiplied by
-    1 + temp_coef * ln(floor((position + 1) / temp_every) + 1) (temp_every 0: not).  Keys go into k_pages, values
+    1 + temp_coef * ln(floor((position + 1) / temp_every) + 1) (temp_every 0: not) and by q_mult.  Keys go into k_pages, values
     (values_are_keys: the keys' columns as projected, and there are no value columns) into v_pages; without pages the
     rows hold queries only.  Returns the queries [T, H * dk] in proj's type."""
     _dev(proj, seq_meta, taps, tails, q_weight, k_weight, inv_freq, slot_mapping, k_pages, v_pages)
@@ -1049,7 +1055,7 @@ def attention_inputs(proj: torch.Tensor, seq_meta: torch.Tensor, num_seqs: int, 
               int(bool(values_are_keys)), _ptr(taps), _code(taps) if taps is not None else 0, int(n_taps),
               _ptr(tails) if n_taps > 1 else None, tails.stride(0) if n_taps > 1 else 0, code, _ptr(q_weight),
               _ptr(k_weight) if own else None, _CODES[w_dtype] if w_dtype is not None else 0, float(eps), _ptr(inv_freq),
-              int(rot_dims), float(temp_coef), int(temp_every), _ptr(seq_meta), int(num_seqs), int(max_q_len),
+              int(rot_dims), float(temp_coef), int(temp_every), float(q_mult), _ptr(seq_meta), int(num_seqs), int(max_q_len),
               _ptr(slot_mapping) if own else None, _ptr(q_out), q_out.stride(0), _ptr(k_pages), _ptr(v_pages) if own else None,
               int(page_size), _stream())
     return q_out

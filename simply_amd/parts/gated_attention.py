@@ -164,14 +164,28 @@ class GatedAttention(Mixer):
         pe = self.position_encoding
         inv_freq, rot_dims = pe.frequencies() if pe is not None else (None, 0)
         coef, every = self.query_temperature if self.query_temperature is not None else (0.0, 0)
+        # the bfloat16 MFMA kernels take values of the keys' size (64, 128 or 256) in pages of a multiple of 16 keys;
+        # they have no factor on the scores, so the queries carry it
+        mfma = dk == dv and proj.dtype == torch.bfloat16 and ops.decode_attention_takes(proj, pages.k_pages, H, 1)
         q = ops.attention_inputs(proj, ctx.seq_meta, ctx.num_seqs, ctx.max_q_len, H, K, dk, dv,
                                  values_are_keys=self.values_are_keys, taps=self.taps, tails=state, norm=self.qk_norm,
                                  q_weight=self.q_norm, k_weight=self.k_norm, eps=self.norm_eps, inv_freq=inv_freq,
-                                 rot_dims=rot_dims, temp_coef=coef, temp_every=every,
+                                 rot_dims=rot_dims, temp_coef=coef, temp_every=every, q_mult=self.scale if mfma else 1.0,
                                  slot_mapping=group.slot_mapping if self.own else None,
                                  k_pages=pages.k_pages if self.own else None, v_pages=pages.v_pages if self.own else None)
-        o = ops.paged_attention_sink(q, pages.k_pages, pages.v_pages, group.block_table, ctx.token_seq, ctx.positions, H,
-                                     scale=self.scale, sinks=self.sinks, slopes=self.slopes, window=self.window)
+        if mfma:
+            o = torch.empty((q.shape[0], H * dv), dtype=q.dtype, device=q.device)
+            units, few, many, max_q = ctx.attention_units(16 // (H // K), ops.prefill_units_per_group())
+            kw = dict(window=self.window, soft_cap=None, max_kv_len=ctx.max_kv_len, max_q_len=max_q, out=o,
+                      sinks=self.sinks, slopes=self.slopes)
+            if few:
+                ops.paged_attention_decode(q, pages.k_pages, pages.v_pages, group.block_table, units, 0, few, H, **kw)
+            if many:
+                ops.paged_attention_prefill(q, pages.k_pages, pages.v_pages, group.block_table, units, few, many, H, **kw)
+        else:
+            o = ops.paged_attention_sink(q, pages.k_pages, pages.v_pages, group.block_table, ctx.token_seq,
+                                         ctx.positions, H, scale=self.scale, sinks=self.sinks, slopes=self.slopes,
+                                         window=self.window)
         if self.output_gate is not None:
             g_at = self.conv_channels
             ops.gated_heads(o, proj[:, g_at:g_at + self.gate_width], H, dv, kind=ops.GATE_SIGMOID, out=o,
