@@ -138,7 +138,7 @@ def _attention_case(dtype, sizes, n, window, page_size, seed=5):
     return q.to(dtype), keys.to(dtype), values.to(dtype), picks
 
 
-def attention_edges(o, device, dtype, page_size=4, n=300, window=37, sizes=(4, 2, 8, 6), scale=0.4):
+def attention_edges(o, device, dtype, page_size=4, n=300, window=37, sizes=(4, 2, 8, 6), scale=0.4, sharp=True):
     """The softmax with one more term exp(0), slopes by distance and a window, by the generic kernel: in a prompt's
     portion (many rows at once) and alone (one row), at the same positions; also without sink and slopes."""
     H, K, dk, dv = sizes
@@ -159,7 +159,7 @@ def attention_edges(o, device, dtype, page_size=4, n=300, window=37, sizes=(4, 2
             for r, i in enumerate(rows):
                 one = o.paged_attention_sink(qrows[r:r + 1], k_pages, v_pages, table, seq[:1], pos[r:r + 1], H, **kw)
                 close(one, want[i:i + 1], tol, f"alone at {i}, window {win}, sink {sink}, slopes {sloped}")
-            if sink and sloped and win is None:
+            if sharp and sink and sloped and win is None:
                 # the comparison is sharp: without the sink, or without the slopes, the answer is another
                 for other in (plain.softmax_attention(q.double(), keys.double(), values.double(), scale, win, slopes, False),
                               plain.softmax_attention(q.double(), keys.double(), values.double(), scale, win, None, True)):

@@ -42,9 +42,9 @@ def test_kernels_with_other_sizes():
         mech.inputs_of_the_first_kind(ops, DEV, dtype, page_size=16, sizes=(4, 2, 32, 16))
         mech.inputs_of_the_second_kind(ops, DEV, dtype, page_size=16, sizes=(4, 4, 64), rot=(64, 10000.0), start=1000)
         mech.inputs_of_the_second_kind(ops, DEV, dtype, page_size=4, sizes=(1, 1, 6), rot=(0, 1.0), start=0)
-        mech.attention_edges(ops, DEV, dtype, page_size=16, sizes=(4, 2, 32, 12))
-        mech.attention_edges(ops, DEV, dtype, page_size=16, sizes=(1, 1, 6, 40), window=64)
-    mech.attention_edges(ops, DEV, torch.float32, page_size=16, sizes=(18, 1, 512, 40))
+        mech.attention_edges(ops, DEV, dtype, page_size=16, sizes=(4, 2, 32, 12), sharp=False)
+        mech.attention_edges(ops, DEV, dtype, page_size=16, sizes=(1, 1, 6, 40), window=64, sharp=False)
+    mech.attention_edges(ops, DEV, torch.float32, page_size=16, sizes=(18, 1, 512, 40), sharp=False)
     mech.inputs_of_the_first_kind(ops, DEV, torch.bfloat16, page_size=16, sizes=(32, 8, 128, 128))
 
 
