@@ -552,6 +552,66 @@ def run_tabupel(args):
             torch.cuda.empty_cache()
 
 
+# --only rudutar: layer sizes that resemble a real model's, for the Rudutar design (layers of the first attention kind
+# in turn with their own keys and values and reading the layer's before them, every third layer of the second kind, all
+# behind windows; dense feed-forwards and routed experts in turn: 16 experts of a quarter of the dense size, two chosen
+# among the two best of four groups, one shared) and, beside it, the closest model that the engine has, Gemma 2 layers
+# behind the same window at equal width, depth, heads and head size, with a gated feed-forward of as many parameters
+RUDUTAR_WINDOW = 1024
+
+
+def rudutar_config(size: dict, layers: int) -> dict:
+    W, H, K, d = size["width"], size["heads"], size["kv_heads"], size["dim"]
+    out, source = [], None
+    for i in range(layers):
+        if i % 2 == 0:
+            mlp = {"kind": "dense", "ff": size["ff"]}
+        else:
+            mlp = {"kind": "moe", "expert": {"ff": size["ff"] // 4}, "shared": {"ff": size["ff"] // 4},
+                   "router": {"experts": 16, "top": 2, "scale": 1.5, "groups": {"count": 4, "keep": 2}}}
+        if i % 3 == 2:
+            out.append({"type": "attention_2", "mlp": mlp,
+                        "mixer": {"heads": H, "kv_heads": K, "dim": d, "vdim": d, "scale": d ** -0.5,
+                                  "mask": {"size": RUDUTAR_WINDOW}, "rot": {"dims": d // 2, "base": 50000.0}}})
+            continue
+        m = {"heads": H, "kv_heads": K, "dim": d, "vdim": d, "scale": d ** -0.5, "conv": 4,
+             "mask": {"size": RUDUTAR_WINDOW}, "q_temp": {"coef": 0.3, "every": 64}}
+        if source is not None:
+            m["kv_from"], source = source, None
+        else:
+            source = i
+        out.append({"type": "attention", "mlp": mlp, "mixer": m})
+    return {"architecture": "Rudutar", "vocab": size["vocab"], "width": W, "norm": {"eps": 1e-6}, "layers": out}
+
+
+def run_rudutar(args):
+    import torch
+    from simply_amd.config import config_from_dict
+    from simply_amd.engine.loading import random_model
+
+    tdtype = torch.bfloat16 if args.dtype == "bfloat16" else torch.float32
+    layers = args.layers or 8
+    for name in args.sizes.split(","):
+        size = ZENUZEN_SIZES[name]
+        gemma = dict(gemma_of_equal_size(size, layers), sliding_window=RUDUTAR_WINDOW,
+                     layer_types=["sliding_attention"] * layers)
+        for label, d in (("rudutar", rudutar_config(size, layers)), ("gemma2-equal-size-windowed", gemma)):
+            if args.alone and label != "rudutar":
+                continue
+            cfg = config_from_dict(d)
+            model = random_model(cfg, 0, tdtype, torch.device("cuda:0"), std=0.02)
+            pt, dt = run_executor_bench(model, size["vocab"], args.prefill_tokens, args.batch, args.context, args.steps,
+                                        args.warmup, args.page_size, args.dtype)
+            print(json.dumps({"metric": "prefill and decode tokens/s through the step function", "model": label,
+                              "size": name, "width": size["width"], "layers": layers,
+                              "prefill_tokens": args.prefill_tokens, "prefill_tokens_per_s": round(args.prefill_tokens / pt, 1),
+                              "prefill_ms": round(pt * 1e3, 3), "batch": args.batch, "context": args.context,
+                              "decode_tokens_per_s": round(args.batch / dt, 1), "decode_ms_per_step": round(dt * 1e3, 3),
+                              "dtype": args.dtype, "data": "synthetic"}), flush=True)
+            del model
+            torch.cuda.empty_cache()
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -567,7 +627,8 @@ def main():
     ap.add_argument("--batches", default="1,8,32,64", help="--only decode-grid: the batch sizes")
     ap.add_argument("--contexts", default="1024,4096,8192", help="--only decode-grid: the context lengths")
     ap.add_argument("--only", default="all", choices=["all", "decode", "decode-grid", "prefill", "prefill-chunked", "products",
-                                                      "gated-products", "ceilings", "zenuzen", "nemidra", "tabupel"],
+                                                      "gated-products", "ceilings", "zenuzen", "nemidra", "tabupel",
+                                                      "rudutar"],
                     help="measure one part alone (for profiles); the line then holds that part only.  products / "
                          "gated-products: the sweep of the product kernels over rows and weight sizes; ceilings: "
                          "what the GPU itself reaches in reading HBM and in bfloat16 MFMA instructions")
@@ -575,8 +636,8 @@ def main():
                     help="decode steps run one at a time after the timed ones, for the p50 and p99 of a step's latency")
     ap.add_argument("--shape", default="2b", choices=sorted(SHAPES), help="layer sizes: Gemma 2 2B (the default), 9B, 27B")
     ap.add_argument("--sizes", default="small,medium,large",
-                    help="--only zenuzen / nemidra / tabupel: which of the layer sizes small, medium, large (8 layers each, or --layers)")
-    ap.add_argument("--alone", action="store_true", help="--only nemidra / tabupel: without the closest model beside it (for profiles)")
+                    help="--only zenuzen / nemidra / tabupel / rudutar: which of the layer sizes small, medium, large (8 layers each, or --layers)")
+    ap.add_argument("--alone", action="store_true", help="--only nemidra / tabupel / rudutar: without the closest model beside it (for profiles)")
     ap.add_argument("--requests", type=int, default=0,
                     help="instead of timed decode steps: a workload of this many requests through the scheduler")
     ap.add_argument("--prompt-min", type=int, default=128)
@@ -608,6 +669,9 @@ def main():
         return
     if args.only == "tabupel":
         run_tabupel(args)
+        return
+    if args.only == "rudutar":
+        run_rudutar(args)
         return
     d = dict(GEMMA2_2B, **SHAPES[args.shape])
     full_layers = d["num_hidden_layers"]

@@ -138,6 +138,140 @@ __global__ __launch_bounds__(kInputThreads) void attention_inputs_kernel(
   }
 }
 
+// The same for bfloat16 rows whose sections are whole pieces of eight entries (key and value sizes that are multiples of
+// 8, rows and pages aligned to 16 bytes): a workgroup takes a token's whole row, a thread eight neighbouring channels at
+// a time, with 16-byte loads of the projection's rows and of the taps and 16-byte stores of queries and keys (a page's
+// key row, in either layout, holds eight neighbouring entries side by side).  The arithmetic, and the order of the
+// convolution's sum, are those of the kernel above; a head's sum of squares is added up from its pieces' sums in their
+// order.
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8v;
+
+__global__ __launch_bounds__(kInputThreads) void attention_inputs_rows_kernel(
+    const bf16* __restrict__ proj, int64_t row_stride, AttentionInputs p, const void* __restrict__ taps, int taps_dtype,
+    const float* __restrict__ tails, int64_t tail_stride, const void* __restrict__ q_w, const void* __restrict__ k_w,
+    int w_dtype, const float* __restrict__ inv_freq, const int* __restrict__ seq_meta,
+    const int64_t* __restrict__ slot_mapping, bf16* __restrict__ q_out, int64_t q_stride, bf16* __restrict__ k_pages,
+    bf16* __restrict__ v_pages, int channels) {
+  extern __shared__ float smem[];
+  float* stage = smem;                      // [channels] the row after the convolution
+  float* piece_ss = stage + channels;       // [channels / 8] sum of squares of every piece
+  __shared__ float red_s[16];
+  const int* meta = seq_meta + 4 * blockIdx.y;
+  const int slot = meta[0], first = meta[1], count = meta[2], pos0 = meta[3];
+  const int j = blockIdx.x;
+  if (j >= count) return;
+  const int t = first + j, pos = pos0 + j, tid = threadIdx.x;
+  const int q_len = p.H * p.dk, k_end = p.k_at + p.K * p.dk;   // (without keys of its own: channels == q_len)
+  const int pieces = channels / 8;
+
+  float ss_q = 0.f, ss_k = 0.f;
+  for (int o = tid; o < pieces; o += kInputThreads) {
+    const int c = o * 8;
+    float v[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = 0.f;
+    if (p.taps >= 1) {
+      const float* tail = tails + static_cast<size_t>(slot) * tail_stride;
+      for (int a = 0; a < p.taps; ++a) {
+        const int jj = j - (p.taps - 1 - a);
+        float u[8];
+        if (jj >= 0) {
+          const bf16x8v x = *reinterpret_cast<const bf16x8v*>(proj + static_cast<size_t>(first + jj) * row_stride + c);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) u[e] = static_cast<float>(x[e]);
+        } else {
+          const float* tp = tail + static_cast<size_t>(p.taps - 1 + jj) * p.conv_channels + c;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) u[e] = tp[e];
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          v[e] = fmaf(load_f(taps, taps_dtype, static_cast<size_t>(c + e) * p.taps + a), u[e], v[e]);
+      }
+    } else {
+      const bf16x8v x = *reinterpret_cast<const bf16x8v*>(proj + static_cast<size_t>(t) * row_stride + c);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = static_cast<float>(x[e]);
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      stage[c + e] = v[e];
+      ss = fmaf(v[e], v[e], ss);
+    }
+    piece_ss[o] = ss;
+    if (c < q_len) ss_q += ss;
+    else if (c < k_end) ss_k += ss;
+  }
+  float r_q = 1.f, r_k = 1.f;
+  if (p.norm == 2) {
+    r_q = 1.f / sqrtf(block_sum(ss_q, red_s) / static_cast<float>(q_len) + p.eps);
+    if (channels > q_len) r_k = 1.f / sqrtf(block_sum(ss_k, red_s) / static_cast<float>(p.K * p.dk) + p.eps);
+  }
+  __syncthreads();
+
+  const bool own = channels > q_len;
+  const int64_t kv_slot = own ? slot_mapping[t] : -1;
+  const int koff = kv_slot >= 0 ? static_cast<int>(kv_slot % p.page_size) : 0;
+  const int64_t page = kv_slot >= 0 ? kv_slot / p.page_size : 0;
+  const float temp = (p.temp_every > 0 ? 1.f + p.temp_coef * logf(static_cast<float>((pos + 1) / p.temp_every) + 1.f) : 1.f) *
+                     p.q_mult;
+  const int half = p.rot_dims / 2;
+  const bool tiled = keys_tiled(p.page_size, p.dk);
+  for (int o = tid; o < pieces; o += kInputThreads) {
+    const int c = o * 8;
+    if (c >= k_end || (c >= q_len && p.values_are_keys)) {
+      // values as they stand (of a layer whose keys are its values: the keys' pieces, before norm and rotation)
+      if (kv_slot >= 0) {
+        const int i = c - (c >= k_end ? p.v_at : p.k_at);
+        const int dv = c >= k_end ? p.dv : p.dk;
+        bf16* dst = v_pages + page * p.K * dv * p.page_size + koff;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) dst[static_cast<size_t>(i + e) * p.page_size] = float_to_bf16(stage[c + e]);
+      }
+      if (c >= k_end) continue;
+    }
+    const bool is_q = c < q_len;
+    if (!is_q && kv_slot < 0) continue;
+    const int base = is_q ? 0 : p.k_at;
+    const int i = c - base, h = i / p.dk, d0 = i % p.dk;
+    const void* w = is_q ? q_w : k_w;
+    float r = 1.f;
+    if (p.norm == 1) {
+      float ss = 0.f;
+      const int po = (base + h * p.dk) / 8;
+      for (int k = 0; k < p.dk / 8; ++k) ss += piece_ss[po + k];
+      r = 1.f / sqrtf(ss / static_cast<float>(p.dk) + p.eps);
+    } else if (p.norm == 2) {
+      r = is_q ? r_q : r_k;
+    }
+    bf16x8v out;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int d = d0 + e;
+      auto normed = [&](int dd) -> float {
+        const float x = stage[base + h * p.dk + dd];
+        if (p.norm == 1) return x * r * load_f(w, w_dtype, dd);
+        if (p.norm == 2) return x * r * load_f(w, w_dtype, h * p.dk + dd);
+        return x;
+      };
+      float x = normed(d);
+      if (d < p.rot_dims) {
+        const float other = normed(d < half ? d + half : d - half);
+        float sn, cs;
+        sincosf(static_cast<float>(pos) * inv_freq[d < half ? d : d - half], &sn, &cs);
+        x = d < half ? x * cs - other * sn : x * cs + other * sn;
+      }
+      out[e] = static_cast<__bf16>(is_q ? x * temp : x);
+    }
+    if (is_q)
+      *reinterpret_cast<bf16x8v*>(q_out + static_cast<size_t>(t) * q_stride + i) = out;
+    else
+      *reinterpret_cast<bf16x8v*>(k_pages + (page * p.K + h) * p.page_size * p.dk +
+                                  key_index(tiled, p.page_size, p.dk, koff, d0)) = out;
+  }
+}
+
 // The tails after the step: the last n - 1 projected rows of every request, from this step's rows and, where the
 // step brought fewer than n - 1 tokens, from the old tail.  A thread takes one channel of one request; it reads old
 // entries only at places that it has not written yet.
@@ -217,6 +351,18 @@ extern "C" int sa_attention_inputs(const void* proj, int dtype, int64_t row_stri
     if (num_taps > 1)
       attention_inputs_tails_kernel<float><<<tail_grid, kWave, 0, stream>>>(static_cast<const float*>(proj), row_stride,
                                                                             num_taps, C, tails, tail_stride, seq_meta);
+  } else if (dk % 8 == 0 && dv % 8 == 0 && row_stride % 8 == 0 && q_stride % 8 == 0 &&
+             reinterpret_cast<uintptr_t>(proj) % 16 == 0 && reinterpret_cast<uintptr_t>(q_out) % 16 == 0 &&
+             reinterpret_cast<uintptr_t>(k_pages) % 16 == 0 &&
+             sizeof(float) * (static_cast<size_t>(C) + C / 8) <= 64 * 1024) {
+    // whole pieces of eight entries, aligned: a workgroup per token, 16-byte accesses
+    attention_inputs_rows_kernel<<<dim3(max_q_len, num_seqs), kInputThreads, sizeof(float) * (C + C / 8), stream>>>(
+        static_cast<const bf16*>(proj), row_stride, p, taps, taps_dtype, tails, tail_stride, q_w, k_w, w_dtype, inv_freq,
+        seq_meta, slot_mapping, static_cast<bf16*>(q_out), q_stride, static_cast<bf16*>(k_pages),
+        static_cast<bf16*>(v_pages), C);
+    if (num_taps > 1)
+      attention_inputs_tails_kernel<bf16><<<tail_grid, kWave, 0, stream>>>(static_cast<const bf16*>(proj), row_stride,
+                                                                           num_taps, C, tails, tail_stride, seq_meta);
   } else {
     attention_inputs_kernel<bf16><<<grid, kInputThreads, smem, stream>>>(
         static_cast<const bf16*>(proj), row_stride, p, taps, taps_dtype, tails, tail_stride, q_w, k_w, w_dtype, inv_freq,
