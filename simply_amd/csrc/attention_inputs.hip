@@ -151,7 +151,8 @@ __global__ __launch_bounds__(kInputThreads) void attention_inputs_rows_kernel(
     const float* __restrict__ tails, int64_t tail_stride, const void* __restrict__ q_w, const void* __restrict__ k_w,
     int w_dtype, const float* __restrict__ inv_freq, const int* __restrict__ seq_meta,
     const int64_t* __restrict__ slot_mapping, bf16* __restrict__ q_out, int64_t q_stride, bf16* __restrict__ k_pages,
-    bf16* __restrict__ v_pages, int channels) {
+    bf16* __restrict__ v_pages, int channels, const bf16* __restrict__ taps_by_tap) {
+  // taps_by_tap (or null): the taps once more as [taps][channels], so that a piece's eight weights of a tap are one load
   extern __shared__ float smem[];
   float* stage = smem;                      // [channels] the row after the convolution
   float* piece_ss = stage + channels;       // [channels / 8] sum of squares of every piece
@@ -184,9 +185,15 @@ __global__ __launch_bounds__(kInputThreads) void attention_inputs_rows_kernel(
 #pragma unroll
           for (int e = 0; e < 8; ++e) u[e] = tp[e];
         }
+        if (taps_by_tap != nullptr) {
+          const bf16x8v wv = *reinterpret_cast<const bf16x8v*>(taps_by_tap + static_cast<size_t>(a) * p.conv_channels + c);
 #pragma unroll
-        for (int e = 0; e < 8; ++e)
-          v[e] = fmaf(load_f(taps, taps_dtype, static_cast<size_t>(c + e) * p.taps + a), u[e], v[e]);
+          for (int e = 0; e < 8; ++e) v[e] = fmaf(static_cast<float>(wv[e]), u[e], v[e]);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            v[e] = fmaf(load_f(taps, taps_dtype, static_cast<size_t>(c + e) * p.taps + a), u[e], v[e]);
+        }
       }
     } else {
       const bf16x8v x = *reinterpret_cast<const bf16x8v*>(proj + static_cast<size_t>(t) * row_stride + c);
@@ -303,7 +310,7 @@ extern "C" int sa_attention_inputs(const void* proj, int dtype, int64_t row_stri
                                    float temp_coef, int temp_every, float q_mult, const int* seq_meta, int num_seqs,
                                    int max_q_len,
                                    const int64_t* slot_mapping, void* q_out, int64_t q_stride, void* k_pages,
-                                   void* v_pages, int page_size, hipStream_t stream) {
+                                   void* v_pages, int page_size, const void* taps_by_tap, hipStream_t stream) {
   if (num_seqs == 0 || max_q_len == 0) return 0;
   const bool own = k_pages != nullptr;   // keys and values of its own (else: queries only)
   SA_REQUIRE(dtype == kF32 || dtype == kBF16, "attention_inputs: unknown dtype %d", dtype);
@@ -359,7 +366,9 @@ extern "C" int sa_attention_inputs(const void* proj, int dtype, int64_t row_stri
     attention_inputs_rows_kernel<<<dim3(max_q_len, num_seqs), kInputThreads, sizeof(float) * (C + C / 8), stream>>>(
         static_cast<const bf16*>(proj), row_stride, p, taps, taps_dtype, tails, tail_stride, q_w, k_w, w_dtype, inv_freq,
         seq_meta, slot_mapping, static_cast<bf16*>(q_out), q_stride, static_cast<bf16*>(k_pages),
-        static_cast<bf16*>(v_pages), C);
+        static_cast<bf16*>(v_pages), C,
+        (taps_dtype == kBF16 && reinterpret_cast<uintptr_t>(taps_by_tap) % 16 == 0) ? static_cast<const bf16*>(taps_by_tap)
+                                                                                    : nullptr);
     if (num_taps > 1)
       attention_inputs_tails_kernel<bf16><<<tail_grid, kWave, 0, stream>>>(static_cast<const bf16*>(proj), row_stride,
                                                                            num_taps, C, tails, tail_stride, seq_meta);

@@ -75,7 +75,7 @@ class GatedAttention(Mixer):
                                   if position_encoding is not None else None)
         if self.position_encoding is not None and not hasattr(self.position_encoding, "frequencies"):
             raise ValueError("gated_attention: the position encoding must give frequencies() (partial_rope)")
-        self.in_proj = self.o_proj = self.in_bias = self.taps = self.q_norm = self.k_norm = None
+        self.in_proj = self.o_proj = self.in_bias = self.taps = self.taps_by_tap = self.q_norm = self.k_norm = None
         self.sinks = self.slopes = None
 
     # ------------------------------------------------------------------ sizes
@@ -132,6 +132,7 @@ class GatedAttention(Mixer):
             self.in_bias = torch.cat([p.to(t["q_bias"].dtype) for p in parts]).contiguous()
         if self.conv_taps >= 1:
             self.taps = torch.cat([t[s + "_conv"] for s in sections], dim=0).contiguous()
+            self.taps_by_tap = self.taps.t().contiguous()   # (what the kernel for aligned rows reads in pieces)
         if self.qk_norm is not None:
             self.q_norm = t["q_norm"].contiguous()
             self.k_norm = t["k_norm"].to(self.q_norm.dtype).contiguous() if self.own else None
@@ -168,7 +169,8 @@ class GatedAttention(Mixer):
         # they have no factor on the scores, so the queries carry it
         mfma = dk == dv and proj.dtype == torch.bfloat16 and ops.decode_attention_takes(proj, pages.k_pages, H, 1)
         q = ops.attention_inputs(proj, ctx.seq_meta, ctx.num_seqs, ctx.max_q_len, H, K, dk, dv,
-                                 values_are_keys=self.values_are_keys, taps=self.taps, tails=state, norm=self.qk_norm,
+                                 values_are_keys=self.values_are_keys, taps=self.taps, taps_by_tap=self.taps_by_tap,
+                                 tails=state, norm=self.qk_norm,
                                  q_weight=self.q_norm, k_weight=self.k_norm, eps=self.norm_eps, inv_freq=inv_freq,
                                  rot_dims=rot_dims, temp_coef=coef, temp_every=every, q_mult=self.scale if mfma else 1.0,
                                  slot_mapping=group.slot_mapping if self.own else None,
