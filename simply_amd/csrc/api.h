@@ -473,12 +473,14 @@ int sa_normalized_readout(const float* x, const float* floor, int64_t floor_stri
 // inv_freq[i], and queries are multiplied by 1 + temp_coef * ln(floor((position + 1) / temp_every) + 1) (temp_every 0:
 // not) and by q_mult.  Queries go to q_out [T, H * dk], keys and values into their pages.  taps_by_tap (or null): the
 // taps once more as [num_taps, channels] in their type, which the kernel for aligned bfloat16 rows reads in pieces.
+// in_bias (or null; only with num_taps 0): a bias per channel that the projection has not had added yet.
 int sa_attention_inputs(const void* proj, int dtype, int64_t row_stride, int H, int K, int dk, int dv, int k_at, int v_at,
                         int values_are_keys, const void* taps, int taps_dtype, int num_taps, float* tails,
                         int64_t tail_stride, int norm, const void* q_w, const void* k_w, int w_dtype, float eps,
                         const float* inv_freq, int rot_dims, float temp_coef, int temp_every, float q_mult,
                         const int* seq_meta, int num_seqs, int max_q_len, const int64_t* slot_mapping, void* q_out, int64_t q_stride,
-                        void* k_pages, void* v_pages, int page_size, const void* taps_by_tap, hipStream_t stream);
+                        void* k_pages, void* v_pages, int page_size, const void* taps_by_tap, const void* in_bias,
+                        int bias_dtype, hipStream_t stream);
 
 // ---- routed experts (routed.hip)
 // softmax over E logits, the top largest: experts [T, top], weights [T, top] = score * scale.

@@ -11,6 +11,7 @@
 //                 position * inv_freq[i]; after the norm.
 //   temperature   queries at position p times 1 + coef * ln(floor((p + 1) / every) + 1)  (every == 0: none), and times
 //                 q_mult (the scores' factor, for an attention kernel that has none of its own).
+//   bias          (without a convolution) a bias per column of the projection, added as the row is read.
 //   values        their own columns of the projection (convolved, otherwise as they are), or the keys' columns as they
 //                 stand before norm and rotation.
 //
@@ -36,6 +37,8 @@ struct AttentionInputs {
   int rot_dims;
   int temp_every;
   float temp_coef, eps;
+  const void* in_bias;      // (or null) added to the projection's columns as they are read; without a convolution only
+  int bias_dtype;
   float q_mult;             // a factor on the queries (the scores' factor, for an attention kernel that has none)
   int page_size;
 };
@@ -76,6 +79,7 @@ __global__ __launch_bounds__(kInputThreads) void attention_inputs_kernel(
       }
     } else {
       v = to_float(row[c]);
+      if (p.in_bias != nullptr) v += load_f(p.in_bias, p.bias_dtype, c);
     }
     stage[i] = v;
   }
@@ -199,6 +203,10 @@ __global__ __launch_bounds__(kInputThreads) void attention_inputs_rows_kernel(
       const bf16x8v x = *reinterpret_cast<const bf16x8v*>(proj + static_cast<size_t>(t) * row_stride + c);
 #pragma unroll
       for (int e = 0; e < 8; ++e) v[e] = static_cast<float>(x[e]);
+      if (p.in_bias != nullptr) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] += load_f(p.in_bias, p.bias_dtype, c + e);
+      }
     }
     float ss = 0.f;
 #pragma unroll
@@ -310,7 +318,8 @@ extern "C" int sa_attention_inputs(const void* proj, int dtype, int64_t row_stri
                                    float temp_coef, int temp_every, float q_mult, const int* seq_meta, int num_seqs,
                                    int max_q_len,
                                    const int64_t* slot_mapping, void* q_out, int64_t q_stride, void* k_pages,
-                                   void* v_pages, int page_size, const void* taps_by_tap, hipStream_t stream) {
+                                   void* v_pages, int page_size, const void* taps_by_tap, const void* in_bias,
+                                   int bias_dtype, hipStream_t stream) {
   if (num_seqs == 0 || max_q_len == 0) return 0;
   const bool own = k_pages != nullptr;   // keys and values of its own (else: queries only)
   SA_REQUIRE(dtype == kF32 || dtype == kBF16, "attention_inputs: unknown dtype %d", dtype);
@@ -325,6 +334,8 @@ extern "C" int sa_attention_inputs(const void* proj, int dtype, int64_t row_stri
              "attention_inputs: %d rotated entries of %d (an even number, with their frequencies)", rot_dims, dk);
   SA_REQUIRE(temp_every >= 0, "attention_inputs: the temperature's period must not be negative");
   SA_REQUIRE(!values_are_keys || dv == dk, "attention_inputs: keys that are the values too have the values' size");
+  SA_REQUIRE(in_bias == nullptr || (num_taps == 0 && (bias_dtype == kF32 || bias_dtype == kBF16)),
+             "attention_inputs: a bias is added here only where no convolution follows (else: before the call)");
   int C = H * dk;
   if (own) {
     SA_REQUIRE(v_pages != nullptr && slot_mapping != nullptr, "attention_inputs: key pages come with value pages and slots");
@@ -348,6 +359,7 @@ extern "C" int sa_attention_inputs(const void* proj, int dtype, int64_t row_stri
   p.H = H, p.K = K, p.dk = dk, p.dv = dv, p.k_at = k_at, p.v_at = v_at, p.values_are_keys = values_are_keys;
   p.taps = num_taps, p.conv_channels = C, p.norm = norm, p.rot_dims = rot_dims, p.temp_every = temp_every;
   p.temp_coef = temp_coef, p.eps = eps, p.page_size = page_size, p.q_mult = q_mult;
+  p.in_bias = in_bias, p.bias_dtype = bias_dtype;
   const dim3 grid(max_q_len, num_seqs, own ? (values_are_keys ? 2 : 3) : 1);
   const dim3 tail_grid((C + kWave - 1) / kWave, num_seqs);
   if (dtype == kF32) {

@@ -94,7 +94,7 @@ _SIGNATURES = {
     "sa_expert_product": [_P, _I, _L, _I, _I, _P, _P, _I, _I, _P, _P, _I, _I, _I, _I, _P, _L, _I, _I, _P],
     "sa_route_choice": [_P, _L, _I, _I, _I, _F, _P, _I, _I, _I, _P, _P, _P],
     "sa_attention_inputs": [_P, _I, _L, _I, _I, _I, _I, _I, _I, _I, _P, _I, _I, _P, _L, _I, _P, _P, _I, _F, _P, _I, _F, _I,
-                            _F, _P, _I, _I, _P, _P, _L, _P, _P, _I, _P, _P],
+                            _F, _P, _I, _I, _P, _P, _L, _P, _P, _I, _P, _P, _I, _P],
     "sa_expert_combine": [_P, _P, _I, _P, _I, _L, _P, _L, _P, _I, _L, _I, _I, _P],
     "sa_sample": [_P, _L, _I, _I, _P, _P, _P, _P, _P, _P, _P, _I, _P, _L, _P],
 }

@@ -996,7 +996,8 @@ def attention_inputs(proj: torch.Tensor, seq_meta: torch.Tensor, num_seqs: int, 
                      taps: torch.Tensor | None = None, tails: torch.Tensor | None = None, norm: str | None = None,
                      q_weight: torch.Tensor | None = None, k_weight: torch.Tensor | None = None, eps: float = 0.0,
                      inv_freq: torch.Tensor | None = None, rot_dims: int = 0, temp_coef: float = 0.0, temp_every: int = 0,
-                     q_mult: float = 1.0, taps_by_tap: torch.Tensor | None = None, slot_mapping: torch.Tensor | None = None, k_pages: torch.Tensor | None = None,
+                     q_mult: float = 1.0, taps_by_tap: torch.Tensor | None = None, in_bias: torch.Tensor | None = None,
+                     slot_mapping: torch.Tensor | None = None, k_pages: torch.Tensor | None = None,
                      v_pages: torch.Tensor | None = None) -> torch.Tensor:
     """From fused projection rows [H * dk queries | K * dk keys | K * dv values | ...] of a ragged step (seq_meta) to
     what an attention kernel reads.  taps [channels, n] with tails float32 [slots, (n - 1) * channels]: every channel
@@ -1007,7 +1008,8 @@ def attention_inputs(proj: torch.Tensor, seq_meta: torch.Tensor, num_seqs: int, 
     1 + temp_coef * ln(floor((position + 1) / temp_every) + 1) (temp_every 0: not) and by q_mult.  Keys go into k_pages, values
     (values_are_keys: the keys' columns as projected, and there are no value columns) into v_pages; without pages the
     rows hold queries only.  taps_by_tap: the taps once more as [n, channels] (what the kernel for aligned bfloat16 rows
-    reads in pieces of eight channels).  Returns the queries [T, H * dk] in proj's type."""
+    reads in pieces of eight channels).  in_bias (only without taps): a bias per channel that the projection has not
+    had added yet.  Returns the queries [T, H * dk] in proj's type."""
     _dev(proj, seq_meta, taps, tails, q_weight, k_weight, inv_freq, slot_mapping, k_pages, v_pages)
     stride = _rows(proj, "attention_inputs: proj")
     T = proj.shape[0]
@@ -1038,7 +1040,9 @@ def attention_inputs(proj: torch.Tensor, seq_meta: torch.Tensor, num_seqs: int, 
     if taps_by_tap is not None and (taps is None or tuple(taps_by_tap.shape) != (n_taps, C) or taps_by_tap.dtype != taps.dtype
                                     or not taps_by_tap.is_contiguous()):
         raise KernelError("attention_inputs: taps_by_tap is the taps transposed, [taps, channels], contiguous")
-    _dev(taps_by_tap)
+    _dev(taps_by_tap, in_bias)
+    if in_bias is not None and (taps is not None or in_bias.numel() < C or not in_bias.is_contiguous()):
+        raise KernelError("attention_inputs: a bias (one entry per channel, contiguous) is added here only without a convolution")
     if rot_dims and (inv_freq is None or inv_freq.dtype != torch.float32 or inv_freq.numel() != rot_dims // 2
                      or not inv_freq.is_contiguous() or rot_dims % 2 or rot_dims > dk):
         raise KernelError("attention_inputs: inv_freq must be float32 [rot_dims / 2], rot_dims even, <= dk")
@@ -1062,7 +1066,7 @@ def attention_inputs(proj: torch.Tensor, seq_meta: torch.Tensor, num_seqs: int, 
               _ptr(k_weight) if own else None, _CODES[w_dtype] if w_dtype is not None else 0, float(eps), _ptr(inv_freq),
               int(rot_dims), float(temp_coef), int(temp_every), float(q_mult), _ptr(seq_meta), int(num_seqs), int(max_q_len),
               _ptr(slot_mapping) if own else None, _ptr(q_out), q_out.stride(0), _ptr(k_pages), _ptr(v_pages) if own else None,
-              int(page_size), _ptr(taps_by_tap), _stream())
+              int(page_size), _ptr(taps_by_tap), _ptr(in_bias), _code(in_bias) if in_bias is not None else 0, _stream())
     return q_out
 
 

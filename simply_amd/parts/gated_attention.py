@@ -160,7 +160,9 @@ class GatedAttention(Mixer):
                                "reads another entry's")
         group = ctx.groups[pages.group_id]
         proj = ops.gemm(x, self.in_proj)
-        if self.bias:
+        # (without a convolution the biases are added where the rows are read; the gate's columns have none)
+        bias_later = self.bias and self.conv_taps == 0
+        if self.bias and not bias_later:
             ops.bias_add_(proj, self.in_bias)
         pe = self.position_encoding
         inv_freq, rot_dims = pe.frequencies() if pe is not None else (None, 0)
@@ -170,6 +172,7 @@ class GatedAttention(Mixer):
         mfma = dk == dv and proj.dtype == torch.bfloat16 and ops.decode_attention_takes(proj, pages.k_pages, H, 1)
         q = ops.attention_inputs(proj, ctx.seq_meta, ctx.num_seqs, ctx.max_q_len, H, K, dk, dv,
                                  values_are_keys=self.values_are_keys, taps=self.taps, taps_by_tap=self.taps_by_tap,
+                                 in_bias=self.in_bias if bias_later else None,
                                  tails=state, norm=self.qk_norm,
                                  q_weight=self.q_norm, k_weight=self.k_norm, eps=self.norm_eps, inv_freq=inv_freq,
                                  rot_dims=rot_dims, temp_coef=coef, temp_every=every, q_mult=self.scale if mfma else 1.0,

@@ -86,7 +86,9 @@ def inputs_of_the_second_kind(o, device, dtype, page_size=4, sizes=(6, 2, 12), r
         padded = torch.cat([torch.zeros((start,) + tuple(v.shape[1:]), dtype=v.dtype), v])
         return plain.rotate_half(padded, dims, base)[start:]
 
+    bias = rand((C,), 14, 0.5).to(dtype)
     xd = x.double()
+    xd[:, :C] += bias.double()
     want_q = at_positions(plain.rms_norm(xd[:, :H * dk], qw.double(), eps).view(n, H, dk))
     want_k = at_positions(plain.rms_norm(xd[:, H * dk:C], kw.double(), eps).view(n, K, dk))
     pages = -(-(start + n) // page_size)
@@ -94,7 +96,7 @@ def inputs_of_the_second_kind(o, device, dtype, page_size=4, sizes=(6, 2, 12), r
     v_pages = torch.full((pages, K, dk, page_size), float("nan"), dtype=dtype, device=device)
     pos = torch.arange(start, start + n)
     q = o.attention_inputs(x.to(device), _meta([[0, 0, n, start]], device), 1, n, H, K, dk, dk, values_are_keys=True,
-                           norm="row", q_weight=qw.to(device), k_weight=kw.to(device), eps=eps,
+                           norm="row", q_weight=qw.to(device), k_weight=kw.to(device), eps=eps, in_bias=bias.to(device),
                            inv_freq=inv_freq.to(device), rot_dims=dims, q_mult=0.5,
                            slot_mapping=pos.to(torch.int64).to(device), k_pages=k_pages, v_pages=v_pages)
     tol = tol_of(dtype)
@@ -103,7 +105,8 @@ def inputs_of_the_second_kind(o, device, dtype, page_size=4, sizes=(6, 2, 12), r
     close(v_pages.cpu()[pos // page_size, :, :, pos % page_size], xd[:, H * dk:C].view(n, K, dk), tol, "values")
     # a layer without keys and values of its own: queries only
     q2 = o.attention_inputs(x.to(device), _meta([[0, 0, n, start]], device), 1, n, H, K, dk, dk, norm="row",
-                            q_weight=qw.to(device), eps=eps, inv_freq=inv_freq.to(device), rot_dims=dims)
+                            q_weight=qw.to(device), eps=eps, inv_freq=inv_freq.to(device), rot_dims=dims,
+                            in_bias=bias[:H * dk].contiguous().to(device))
     close(q2.view(n, H, dk), want_q, tol, "queries alone")
 
 
@@ -207,7 +210,22 @@ def attention_on_the_matrix_cores(o, device, sizes=(8, 2, 64, 64), n=700, window
         close(out2, want, 4e-2, f"units of a portion, sink {sink}")
 
 
-# --------------------------------------------------------------------------- gates, router, experts
+# --------------------------------------------------------------------------- embedding, gates, router, experts
+
+
+def normed_embedding(device, dtype):
+    """The table's row through the norm with a weight of its own, 32-bit out."""
+    from simply_amd import registry
+
+    V, D, eps = 37, 24, 1e-3
+    table, w = rand((V, D), 1, 3.0).to(dtype), rand((D,), 2).to(dtype)
+    part = registry.EMBEDDINGS.build("normed_embedding", vocab_size=V, dim=D, eps=eps)
+    part.load({"table": table.to(device), "norm": w.to(device)})
+    tokens = torch.tensor([0, 36, 5, 5, 17], dtype=torch.int32, device=device)
+    got = part.forward(tokens)
+    assert got.dtype == torch.float32
+    close(got, plain.rms_norm(table.double()[tokens.cpu().long()], w.double(), eps), 2e-6, "normed rows")
+
 
 
 def gate_per_head(o, device, dtype):

@@ -28,6 +28,11 @@ def test_kernel(body, dtype):
     body(ops, DEV, dtype)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_normed_embedding(dtype):
+    mech.normed_embedding(DEV, dtype)
+
+
 def test_router():
     mech.router_choice(ops, DEV)
     mech.router_choice(ops, DEV, torch.bfloat16)    # (a correction stored in bfloat16)

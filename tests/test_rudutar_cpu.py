@@ -112,6 +112,11 @@ def test_reference_of_a_kernel(body, dtype):
     body(torch_ops, CPU, dtype)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_normed_embedding(cpu_ops, dtype):
+    mech.normed_embedding(CPU, dtype)
+
+
 def test_router_reference():
     mech.router_choice(torch_ops, CPU)
 

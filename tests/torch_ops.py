@@ -780,13 +780,15 @@ def rglru_scan(u, gates, block, r_bias, i_bias, lam, y, y_bias, state, seq_meta,
 
 def attention_inputs(proj, seq_meta, num_seqs, max_q_len, num_heads, num_kv_heads, key_dim, value_dim, *,
                      values_are_keys=False, taps=None, tails=None, norm=None, q_weight=None, k_weight=None, eps=0.0,
-                     inv_freq=None, rot_dims=0, temp_coef=0.0, temp_every=0, q_mult=1.0, taps_by_tap=None,
+                     inv_freq=None, rot_dims=0, temp_coef=0.0, temp_every=0, q_mult=1.0, taps_by_tap=None, in_bias=None,
                      slot_mapping=None, k_pages=None, v_pages=None):
     H, K, dk, dv = num_heads, num_kv_heads, key_dim, value_dim
     own = k_pages is not None
     C = (H + K) * dk + (0 if values_are_keys else K * dv) if own else H * dk
     T = proj.shape[0]
     x = _f(proj[:, :C]).clone()
+    if in_bias is not None:
+        x = x + _f(in_bias)[:C]
     if taps is not None:
         n, w = taps.shape[1], _f(taps)
         for slot, first, count, _ in seq_meta[:num_seqs].tolist():
