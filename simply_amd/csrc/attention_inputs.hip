@@ -53,6 +53,7 @@ __global__ __launch_bounds__(kInputThreads) void attention_inputs_kernel(
   extern __shared__ float smem[];
   float* stage = smem;                 // [stage_len] the section after the convolution
   float* head_r = stage + stage_len;   // [heads] 1 / rms of every head (norm 1)
+  float* rot_s = head_r + (p.H > p.K ? p.H : p.K);   // [rot_dims] the token's cosines, then its sines
   __shared__ float red_s[16];
   const int* meta = seq_meta + 4 * blockIdx.y;
   const int slot = meta[0], first = meta[1], count = meta[2], pos0 = meta[3];
@@ -83,6 +84,9 @@ __global__ __launch_bounds__(kInputThreads) void attention_inputs_kernel(
     }
     stage[i] = v;
   }
+  // the token's angles once for all heads (every head turns by the same ones)
+  for (int i = tid; i < p.rot_dims / 2; i += kInputThreads)
+    sincosf(static_cast<float>(pos) * inv_freq[i], &rot_s[p.rot_dims / 2 + i], &rot_s[i]);
   __syncthreads();
 
   const int64_t kv_slot = sec > 0 ? slot_mapping[t] : -1;
@@ -131,8 +135,7 @@ __global__ __launch_bounds__(kInputThreads) void attention_inputs_kernel(
     float v = normed(h, d);
     if (d < p.rot_dims) {
       const float o = normed(h, d < half ? d + half : d - half);
-      float sn, cs;
-      sincosf(static_cast<float>(pos) * inv_freq[d < half ? d : d - half], &sn, &cs);
+      const float cs = rot_s[d < half ? d : d - half], sn = rot_s[half + (d < half ? d : d - half)];
       v = d < half ? v * cs - o * sn : v * cs + o * sn;
     }
     if (sec == 0)
@@ -160,6 +163,7 @@ __global__ __launch_bounds__(kInputThreads) void attention_inputs_rows_kernel(
   extern __shared__ float smem[];
   float* stage = smem;                      // [channels] the row after the convolution
   float* piece_ss = stage + channels;       // [channels / 8] sum of squares of every piece
+  float* rot_s = piece_ss + channels / 8;   // [rot_dims] the token's cosines, then its sines
   __shared__ float red_s[16];
   const int* meta = seq_meta + 4 * blockIdx.y;
   const int slot = meta[0], first = meta[1], count = meta[2], pos0 = meta[3];
@@ -218,6 +222,8 @@ __global__ __launch_bounds__(kInputThreads) void attention_inputs_rows_kernel(
     if (c < q_len) ss_q += ss;
     else if (c < k_end) ss_k += ss;
   }
+  for (int i = tid; i < p.rot_dims / 2; i += kInputThreads)
+    sincosf(static_cast<float>(pos) * inv_freq[i], &rot_s[p.rot_dims / 2 + i], &rot_s[i]);
   float r_q = 1.f, r_k = 1.f;
   if (p.norm == 2) {
     r_q = 1.f / sqrtf(block_sum(ss_q, red_s) / static_cast<float>(q_len) + p.eps);
@@ -273,8 +279,7 @@ __global__ __launch_bounds__(kInputThreads) void attention_inputs_rows_kernel(
       float x = normed(d);
       if (d < p.rot_dims) {
         const float other = normed(d < half ? d + half : d - half);
-        float sn, cs;
-        sincosf(static_cast<float>(pos) * inv_freq[d < half ? d : d - half], &sn, &cs);
+        const float cs = rot_s[d < half ? d : d - half], sn = rot_s[half + (d < half ? d : d - half)];
         x = d < half ? x * cs - other * sn : x * cs + other * sn;
       }
       out[e] = static_cast<__bf16>(is_q ? x * temp : x);
@@ -353,7 +358,7 @@ extern "C" int sa_attention_inputs(const void* proj, int dtype, int64_t row_stri
   int stage_len = H * dk;
   if (own && K * dk > stage_len) stage_len = K * dk;
   if (own && !values_are_keys && K * dv > stage_len) stage_len = K * dv;
-  const size_t smem = sizeof(float) * (static_cast<size_t>(stage_len) + max_heads);
+  const size_t smem = sizeof(float) * (static_cast<size_t>(stage_len) + max_heads + rot_dims);
   SA_REQUIRE(smem <= 64 * 1024, "attention_inputs: rows of %d entries do not fit a workgroup's LDS", stage_len);
   AttentionInputs p;
   p.H = H, p.K = K, p.dk = dk, p.dv = dv, p.k_at = k_at, p.v_at = v_at, p.values_are_keys = values_are_keys;
@@ -373,9 +378,10 @@ extern "C" int sa_attention_inputs(const void* proj, int dtype, int64_t row_stri
   } else if (dk % 8 == 0 && dv % 8 == 0 && row_stride % 8 == 0 && q_stride % 8 == 0 &&
              reinterpret_cast<uintptr_t>(proj) % 16 == 0 && reinterpret_cast<uintptr_t>(q_out) % 16 == 0 &&
              reinterpret_cast<uintptr_t>(k_pages) % 16 == 0 &&
-             sizeof(float) * (static_cast<size_t>(C) + C / 8) <= 64 * 1024) {
+             sizeof(float) * (static_cast<size_t>(C) + C / 8 + rot_dims) <= 64 * 1024) {
     // whole pieces of eight entries, aligned: a workgroup per token, 16-byte accesses
-    attention_inputs_rows_kernel<<<dim3(max_q_len, num_seqs), kInputThreads, sizeof(float) * (C + C / 8), stream>>>(
+    attention_inputs_rows_kernel<<<dim3(max_q_len, num_seqs), kInputThreads, sizeof(float) * (C + C / 8 + rot_dims),
+                                   stream>>>(
         static_cast<const bf16*>(proj), row_stride, p, taps, taps_dtype, tails, tail_stride, q_w, k_w, w_dtype, inv_freq,
         seq_meta, slot_mapping, static_cast<bf16*>(q_out), q_stride, static_cast<bf16*>(k_pages),
         static_cast<bf16*>(v_pages), C,
