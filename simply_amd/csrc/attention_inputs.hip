@@ -39,6 +39,7 @@ struct AttentionInputs {
   float temp_coef, eps;
   const void* in_bias;      // (or null) added to the projection's columns as they are read; without a convolution only
   int bias_dtype;
+  int own_tails;            // every request brings one token: the thread that reads a channel's tail also moves it on
   float q_mult;             // a factor on the queries (the scores' factor, for an attention kernel that has none)
   int page_size;
 };
@@ -46,7 +47,7 @@ struct AttentionInputs {
 template <typename T>
 __global__ __launch_bounds__(kInputThreads) void attention_inputs_kernel(
     const T* __restrict__ proj, int64_t row_stride, AttentionInputs p, const void* __restrict__ taps, int taps_dtype,
-    const float* __restrict__ tails, int64_t tail_stride, const void* __restrict__ q_w, const void* __restrict__ k_w,
+    float* __restrict__ tails, int64_t tail_stride, const void* __restrict__ q_w, const void* __restrict__ k_w,
     int w_dtype, const float* __restrict__ inv_freq, const int* __restrict__ seq_meta,
     const int64_t* __restrict__ slot_mapping, T* __restrict__ q_out, int64_t q_stride, T* __restrict__ k_pages,
     T* __restrict__ v_pages, int stage_len) {
@@ -70,13 +71,15 @@ __global__ __launch_bounds__(kInputThreads) void attention_inputs_kernel(
     const int c = col0 + i;
     float v;
     if (p.taps >= 1) {
-      const float* tail = tails + static_cast<size_t>(slot) * tail_stride;
+      float* tail = tails + static_cast<size_t>(slot) * tail_stride;
       v = 0.f;
       for (int a = 0; a < p.taps; ++a) {
         const int jj = j - (p.taps - 1 - a);   // the request's token of this step under tap a; negative: an earlier step's
         const float u = jj >= 0 ? to_float(proj[static_cast<size_t>(first + jj) * row_stride + c])
                                 : tail[static_cast<size_t>(p.taps - 1 + jj) * p.conv_channels + c];
         v = fmaf(load_f(taps, taps_dtype, static_cast<size_t>(c) * p.taps + a), u, v);
+        // (one token a request: what tap a read is the tail's entry a - 1 from now on; entry a - 1 has been read)
+        if (p.own_tails && a >= 1) tail[static_cast<size_t>(a - 1) * p.conv_channels + c] = u;
       }
     } else {
       v = to_float(row[c]);
@@ -155,7 +158,7 @@ typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8v;
 
 __global__ __launch_bounds__(kInputThreads) void attention_inputs_rows_kernel(
     const bf16* __restrict__ proj, int64_t row_stride, AttentionInputs p, const void* __restrict__ taps, int taps_dtype,
-    const float* __restrict__ tails, int64_t tail_stride, const void* __restrict__ q_w, const void* __restrict__ k_w,
+    float* __restrict__ tails, int64_t tail_stride, const void* __restrict__ q_w, const void* __restrict__ k_w,
     int w_dtype, const float* __restrict__ inv_freq, const int* __restrict__ seq_meta,
     const int64_t* __restrict__ slot_mapping, bf16* __restrict__ q_out, int64_t q_stride, bf16* __restrict__ k_pages,
     bf16* __restrict__ v_pages, int channels, const bf16* __restrict__ taps_by_tap) {
@@ -180,7 +183,7 @@ __global__ __launch_bounds__(kInputThreads) void attention_inputs_rows_kernel(
 #pragma unroll
     for (int e = 0; e < 8; ++e) v[e] = 0.f;
     if (p.taps >= 1) {
-      const float* tail = tails + static_cast<size_t>(slot) * tail_stride;
+      float* tail = tails + static_cast<size_t>(slot) * tail_stride;
       for (int a = 0; a < p.taps; ++a) {
         const int jj = j - (p.taps - 1 - a);
         float u[8];
@@ -192,6 +195,11 @@ __global__ __launch_bounds__(kInputThreads) void attention_inputs_rows_kernel(
           const float* tp = tail + static_cast<size_t>(p.taps - 1 + jj) * p.conv_channels + c;
 #pragma unroll
           for (int e = 0; e < 8; ++e) u[e] = tp[e];
+        }
+        if (p.own_tails && a >= 1) {   // (one token a request: what tap a read is the tail's entry a - 1 from now on)
+          float* tw = tail + static_cast<size_t>(a - 1) * p.conv_channels + c;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) tw[e] = u[e];
         }
         if (taps_by_tap != nullptr) {
           const bf16x8v wv = *reinterpret_cast<const bf16x8v*>(taps_by_tap + static_cast<size_t>(a) * p.conv_channels + c);
@@ -365,6 +373,9 @@ extern "C" int sa_attention_inputs(const void* proj, int dtype, int64_t row_stri
   p.taps = num_taps, p.conv_channels = C, p.norm = norm, p.rot_dims = rot_dims, p.temp_every = temp_every;
   p.temp_coef = temp_coef, p.eps = eps, p.page_size = page_size, p.q_mult = q_mult;
   p.in_bias = in_bias, p.bias_dtype = bias_dtype;
+  // with one token a request a channel's tail has one reader, who moves it on; else a second launch does, behind all readers
+  p.own_tails = max_q_len == 1 && num_taps > 1;
+  const bool tails_launch = num_taps > 1 && !p.own_tails;
   const dim3 grid(max_q_len, num_seqs, own ? (values_are_keys ? 2 : 3) : 1);
   const dim3 tail_grid((C + kWave - 1) / kWave, num_seqs);
   if (dtype == kF32) {
@@ -372,7 +383,7 @@ extern "C" int sa_attention_inputs(const void* proj, int dtype, int64_t row_stri
         static_cast<const float*>(proj), row_stride, p, taps, taps_dtype, tails, tail_stride, q_w, k_w, w_dtype, inv_freq,
         seq_meta, slot_mapping, static_cast<float*>(q_out), q_stride, static_cast<float*>(k_pages),
         static_cast<float*>(v_pages), stage_len);
-    if (num_taps > 1)
+    if (tails_launch)
       attention_inputs_tails_kernel<float><<<tail_grid, kWave, 0, stream>>>(static_cast<const float*>(proj), row_stride,
                                                                             num_taps, C, tails, tail_stride, seq_meta);
   } else if (dk % 8 == 0 && dv % 8 == 0 && row_stride % 8 == 0 && q_stride % 8 == 0 &&
@@ -387,7 +398,7 @@ extern "C" int sa_attention_inputs(const void* proj, int dtype, int64_t row_stri
         static_cast<bf16*>(v_pages), C,
         (taps_dtype == kBF16 && reinterpret_cast<uintptr_t>(taps_by_tap) % 16 == 0) ? static_cast<const bf16*>(taps_by_tap)
                                                                                     : nullptr);
-    if (num_taps > 1)
+    if (tails_launch)
       attention_inputs_tails_kernel<bf16><<<tail_grid, kWave, 0, stream>>>(static_cast<const bf16*>(proj), row_stride,
                                                                            num_taps, C, tails, tail_stride, seq_meta);
   } else {
@@ -395,7 +406,7 @@ extern "C" int sa_attention_inputs(const void* proj, int dtype, int64_t row_stri
         static_cast<const bf16*>(proj), row_stride, p, taps, taps_dtype, tails, tail_stride, q_w, k_w, w_dtype, inv_freq,
         seq_meta, slot_mapping, static_cast<bf16*>(q_out), q_stride, static_cast<bf16*>(k_pages),
         static_cast<bf16*>(v_pages), stage_len);
-    if (num_taps > 1)
+    if (tails_launch)
       attention_inputs_tails_kernel<bf16><<<tail_grid, kWave, 0, stream>>>(static_cast<const bf16*>(proj), row_stride,
                                                                            num_taps, C, tails, tail_stride, seq_meta);
   }
