@@ -14,7 +14,9 @@
 // and simply/kernels/ragged_paged_attention.py:222-249; query head h reads
 // key/value head h / G (simply/kernels/ragged_paged_attention.py:214-215).
 //
-// Three options for mixers that are not plain softmax attention:
+// Options for mixers that are not plain softmax attention:
+//   slopes           a bias by distance: slopes[h] * (query position - key position) is taken off head h's scaled scores
+//                    (with sinks, below the entry points: one more term exp(sinks[h]) in the sum, without a value).
 //   maps (M > 1)     every query head has M score maps over the same values: its query row is M vectors of hd
 //                    entries, a key row M * hd entries (one key vector per map); each map is a softmax of its own.
 //                    To the kernel a map is one more query head ("virtual head" g = head * M + map).
